@@ -1,0 +1,116 @@
+"""Writes the golden vectors under tests/golden/ from the reference's own CPU
+MoE implementation.
+
+Run in a container that has the reference checkout: ``make -C oracle ref``
+compiles the reference's header-only CPU MoE (from where it lies, nothing is
+copied) into oracle/_ref/libref_moe.so; this script calls it on seeded inputs
+and stores inputs-by-seed plus expected outputs as small .npz files. The
+fixtures, not the reference, travel with the repository.
+
+    python tests/golden/make_golden.py
+"""
+import hashlib
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+
+from flash_distributed_moe_amd import synth  # noqa: E402
+from oracle import oracle  # noqa: E402
+
+
+def digest(*arrays):
+    h = hashlib.sha256()
+    for a in arrays:
+        h.update(np.ascontiguousarray(a).tobytes())
+    return np.frombuffer(h.digest(), dtype=np.uint8).copy()
+
+
+SMALL_SHAPES = [
+    # name, T, H, E, k, I, dtype, seed
+    ("s0", 5, 64, 16, 4, 32, "f32", 11),
+    ("s1", 7, 96, 8, 8, 48, "f32", 12),      # k == E: every expert selected
+    ("s2", 3, 128, 32, 1, 16, "bf16", 13),   # top-1
+    ("s3", 9, 256, 64, 6, 64, "bf16", 14),
+]
+
+
+def main():
+    if not oracle.have_ref():
+        oracle.build(ref=True)
+
+    # 1. BASELINE config 1 (tiny fp32), whole layer.
+    cfg = synth.CONFIGS["tiny_f32"]
+    inp = synth.make_inputs_np(cfg, seed=7907)
+    out = oracle.ref_full_moe(inp["tokens"], inp["gate"], inp["ffn1"], inp["ffn2"], cfg.k)
+    idx, w = oracle.ref_moe_gate(inp["tokens"], inp["gate"], cfg.k)
+    np.savez_compressed(os.path.join(HERE, "ref_tiny_f32.npz"), seed=7907, out=out,
+                        topk_idx=idx, topk_w=w,
+                        input_digest=digest(inp["tokens"], inp["gate"], inp["ffn1"], inp["ffn2"]))
+
+    # 2. Small odd shapes, whole layer and router.
+    pack = {}
+    for name, T, H, E, k, I, dt, seed in SMALL_SHAPES:
+        c = synth.MoeConfig(name, T, H, E, k, I, dt)
+        inp = synth.make_inputs_np(c, seed=seed)
+        pack[name + "_out"] = oracle.ref_full_moe(inp["tokens"], inp["gate"], inp["ffn1"],
+                                                  inp["ffn2"], k)
+        i2, w2 = oracle.ref_moe_gate(inp["tokens"], inp["gate"], k)
+        pack[name + "_idx"], pack[name + "_w"] = i2, w2
+        pack[name + "_digest"] = digest(inp["tokens"], inp["gate"], inp["ffn1"], inp["ffn2"])
+    np.savez_compressed(os.path.join(HERE, "ref_small_shapes.npz"), **pack)
+
+    # 3. Router at the Qwen3-30B-A3B router shape (E128, H2048, top-8), bf16-valued
+    #    inputs, 32 tokens.
+    c = synth.CONFIGS["qwen3_30b_decode"]
+    gate = synth.normal_np(7907, synth.STREAM_GATE, (c.E, c.H), synth.SIGMA_W, True)
+    x = synth.normal_np(7907, synth.STREAM_TOKENS, (32, c.H), synth.SIGMA_X, True)
+    i3, w3 = oracle.ref_moe_gate(x, gate, c.k)
+    np.savez_compressed(os.path.join(HERE, "ref_gate_30b.npz"), seed=7907, topk_idx=i3,
+                        topk_w=w3, input_digest=digest(x, gate))
+
+    # 4. Top-k tie / NaN / short-row behaviour and softmax rows.
+    nan = np.float32("nan")
+    tie_rows = np.array([
+        [1, 3, 3, 0, 3, 1, 1, -2],
+        [5, 5, 5, 5, 5, 5, 5, 5],
+        [0, -1, nan, 7, 7, nan, 2, 2],
+        [-3, -3, -2, -2, -1, -1, 0, 0],
+        [nan, nan, nan, nan, nan, nan, nan, nan],
+        [np.float32("inf"), 1, np.float32("-inf"), np.float32("inf"), 0, 0, 9, 9],
+    ], dtype=np.float32)
+    tv, ti = oracle.ref_topk(tie_rows, 4)
+    short = np.array([[2, 9, 2], [1, 1, 1]], dtype=np.float32)
+    sv, si = oracle.ref_topk(short, 5)          # cols < k: unfilled slots
+    sm_in = np.array([[0, 0, 0, 0], [1, 2, 3, 4], [-50, 0, 50, 100], [88, 88.5, -88, 3],
+                      [1e-3, -1e-3, 0, 5e-4]], dtype=np.float32)
+    sm = oracle.ref_softmax_rows(sm_in)
+    np.savez_compressed(os.path.join(HERE, "ref_topk_softmax_cases.npz"), tie_rows=tie_rows,
+                        tie_vals=tv, tie_idx=ti, short_rows=short, short_vals=sv, short_idx=si,
+                        softmax_in=sm_in, softmax_out=sm)
+
+    # 5. The reference's own test input recipe (srand(7907), rand()), small shape.
+    T, E, H, I, k = 6, 8, 128, 64, 3
+    tok, g, f1, f2 = oracle.reference_test_inputs(T, E, H, I, seed=7907)
+    o5 = oracle.ref_full_moe(tok, g, f1, f2, k)
+    np.savez_compressed(os.path.join(HERE, "ref_rand_inputs_small.npz"), T=T, E=E, H=H, I=I,
+                        k=k, out=o5, input_digest=digest(tok, g, f1, f2))
+
+    # 6. SiLU*up stage alone (refExpertFFN1).
+    c = synth.MoeConfig("ffn1", 4, 64, 1, 1, 24, "f32")
+    inp = synth.make_inputs_np(c, seed=21)
+    big = inp["tokens"] * np.float32(40.0)       # push pre-activations into both sigmoid branches
+    w13 = inp["ffn1"][0] * np.float32(20.0)
+    np.savez_compressed(os.path.join(HERE, "ref_ffn1.npz"), seed=21,
+                        out=oracle.ref_expert_ffn1(big, w13))
+    for f in sorted(os.listdir(HERE)):
+        if f.endswith(".npz"):
+            print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")
+
+
+if __name__ == "__main__":
+    main()
