@@ -1,0 +1,56 @@
+"""Builds libflashMoe.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+    python -m flash_distributed_moe_amd.build
+"""
+import glob
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libflashMoe.so")
+
+# -packed-fp32-ops: keep the compiler from forming packed float32 instructions.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-DNDEBUG",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-return-type-c-linkage",
+]
+
+
+def sources():
+    return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+
+
+def build(verbose=True):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    os.makedirs(LIB_DIR, exist_ok=True)
+    objs = []
+    procs = []
+    for src in sources():
+        obj = os.path.join(LIB_DIR, os.path.basename(src) + ".o")
+        objs.append(obj)
+        cmd = [hipcc] + HIPCC_FLAGS + ["-c", src, "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((cmd, subprocess.Popen(cmd, stderr=subprocess.PIPE, text=True)))
+    for cmd, p in procs:
+        _, err = p.communicate()
+        err = "\n".join(l for l in err.splitlines() if "packed-fp32-ops" not in l)
+        if p.returncode != 0:
+            sys.stderr.write(err + "\n")
+            raise RuntimeError("hipcc failed: " + " ".join(cmd))
+        if verbose and err.strip():
+            sys.stderr.write(err + "\n")
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs + [
+        "-Wl,--version-script=" + os.path.join(CSRC, "lib.version"), "-Wl,-soname,libflashMoe.so"]
+    if verbose:
+        print(" ".join(link), flush=True)
+    subprocess.check_call(link)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build())

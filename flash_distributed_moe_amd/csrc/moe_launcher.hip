@@ -1,0 +1,391 @@
+// Host side of libflashMoe.so: workspace layout, validation, launch, the C ABI
+// of include/flash_moe.h and the C++ interface of include/iMoeKernelLauncher.h.
+//
+// Differences from the reference's host launcher
+// (src/hip/launcher/moeKernelLauncher.hip:58-212) that matter to callers:
+//  * shape, dtype and top-k are run-time fields, not compile-time constants
+//  * all per-launcher state travels in the kernel argument, so any number of
+//    launchers can live on one device (the reference keeps its state in
+//    process-global __constant__ symbols)
+//  * a launch issues exactly one kernel and no memset/memcpy: the kernel
+//    returns its counters to zero itself, which also makes a launch capturable
+//    in a HIP graph
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "../../include/iMoeKernelLauncher.h"
+#include "moe_params.h"
+
+namespace fmoe {
+hipError_t launch_stream_kernel(const Params& p, int dtype, int grid, hipStream_t stream);
+}
+
+#define FMOE_FILENAME (strrchr(__FILE__, '/') ? strrchr(__FILE__, '/') + 1 : __FILE__)
+
+// Same convention as the reference (src/hip/hipHostCommon.h:11-19): print to
+// stdout, return the first failing code.
+#define FMOE_HIP_CHECK(expr)                                               \
+  do {                                                                     \
+    const hipError_t fmoe_err_ = (expr);                                   \
+    if (fmoe_err_ != hipSuccess) {                                         \
+      printf("[MOE HIP ERROR: %s:%i]: %s\n", FMOE_FILENAME, __LINE__,      \
+             hipGetErrorString(fmoe_err_));                                \
+      return fmoe_err_;                                                    \
+    }                                                                      \
+  } while (0)
+
+#define FMOE_FAIL(code, fmt, ...)                                                      \
+  do {                                                                                 \
+    printf("[MOE ERROR: %s:%i]: " fmt "\n", FMOE_FILENAME, __LINE__, ##__VA_ARGS__);   \
+    return (code);                                                                     \
+  } while (0)
+
+namespace {
+
+constexpr long long kMaxRows = 1ll << 21;  // max_tokens * top_k a launcher may be sized for
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct Layout {
+  size_t ctl, g1_done, topk_idx, topk_w, masks, word_prefix, expert_count, expert_offset, perm,
+      row_w, mtiles, h, y, total;
+  size_t zero_bytes;  // leading region that must be zero before a launch
+  int W, max_mtiles;
+};
+
+Layout make_layout(const FlashMoeLayerDesc& d) {
+  Layout L{};
+  const size_t rows = static_cast<size_t>(d.max_tokens) * d.top_k;
+  const size_t esz = d.dtype == FLASH_MOE_BF16 ? 2 : 4;
+  L.W = (d.max_tokens + 63) / 64;
+  L.max_mtiles = static_cast<int>((rows + fmoe::SKINNY_MT - 1) / fmoe::SKINNY_MT) + d.experts;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = off;
+    off = align_up(off + bytes, 256);
+    return at;
+  };
+  // zero-initialised region first: control block, per-tile counters, masks
+  L.ctl = take(sizeof(fmoe::Control));
+  L.g1_done = take(sizeof(unsigned) * L.max_mtiles);
+  L.masks = take(sizeof(unsigned long long) * d.experts * L.W);
+  L.zero_bytes = off;
+  L.word_prefix = take(sizeof(int) * d.experts * L.W);
+  L.topk_idx = take(sizeof(int) * rows);
+  L.topk_w = take(sizeof(float) * rows);
+  L.expert_count = take(sizeof(int) * d.experts);
+  L.expert_offset = take(sizeof(int) * (d.experts + 1));
+  L.perm = take(sizeof(int) * rows);
+  L.row_w = take(sizeof(float) * rows);
+  L.mtiles = take(sizeof(fmoe::TileDesc) * L.max_mtiles);
+  L.h = take(esz * rows * d.intermediate);
+  L.y = take(sizeof(float) * rows * d.hidden);
+  L.total = off;
+  return L;
+}
+
+hipError_t validate(const FlashMoeLayerDesc* d) {
+  if (d == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null layer description");
+  if (d->dtype != FLASH_MOE_F32 && d->dtype != FLASH_MOE_BF16)
+    FMOE_FAIL(hipErrorInvalidValue, "dtype %i is neither float32 (0) nor bfloat16 (1)", d->dtype);
+  if (d->experts < 1 || d->experts > fmoe::MAX_EXPERTS)
+    FMOE_FAIL(hipErrorInvalidValue, "experts = %i, supported 1..%i", d->experts,
+              fmoe::MAX_EXPERTS);
+  if (d->top_k < 1 || d->top_k > d->experts || d->top_k > fmoe::MAX_TOPK)
+    FMOE_FAIL(hipErrorInvalidValue, "top_k = %i, supported 1..min(experts, %i)", d->top_k,
+              fmoe::MAX_TOPK);
+  if (d->hidden < 64 || d->hidden % 64 != 0)
+    FMOE_FAIL(hipErrorInvalidValue, "hidden = %i must be a positive multiple of 64", d->hidden);
+  if (d->intermediate < 32 || d->intermediate % 32 != 0)
+    FMOE_FAIL(hipErrorInvalidValue, "intermediate = %i must be a positive multiple of 32",
+              d->intermediate);
+  if (d->max_tokens < 1) FMOE_FAIL(hipErrorInvalidValue, "max_tokens = %i", d->max_tokens);
+  // Capacity comes before any pointer is looked at, as in the reference
+  // (src/hip/launcher/moeKernelLauncher.hip:117-135; pinned there by
+  // test/singleGPU/cpp/moe/moeApiTest.cpp:5-12 with null weights).
+  if (static_cast<long long>(d->max_tokens) * d->top_k > kMaxRows)
+    FMOE_FAIL(hipErrorUnknown,
+              "max_tokens = %i is beyond capacity: this configuration handles %lli tokens",
+              d->max_tokens, kMaxRows / d->top_k);
+  if (d->sched < FLASH_MOE_SCHED_AUTO || d->sched > FLASH_MOE_SCHED_TILED)
+    FMOE_FAIL(hipErrorInvalidValue, "sched = %i", d->sched);
+  return hipSuccess;
+}
+
+}  // namespace
+
+struct FlashMoeLauncher {
+  FlashMoeLayerDesc desc;
+  Layout layout;
+  char* ws = nullptr;
+  int device = 0;
+  int num_cus = 0;
+  long long ticks_per_ms = 100000;
+  long long spin_limit = 0;
+  int last_tokens = 0;
+};
+
+namespace {
+
+fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* output, int T) {
+  const FlashMoeLayerDesc& d = l->desc;
+  const Layout& L = l->layout;
+  fmoe::Params p{};
+  p.T = T;
+  p.E = d.experts;
+  p.H = d.hidden;
+  p.K = d.top_k;
+  p.I = d.intermediate;
+  p.W = L.W;
+  p.n_workers = l->num_cus * 8;
+  p.max_mtiles = L.max_mtiles;
+  p.spin_limit = l->spin_limit;
+  p.tokens = tokens;
+  p.gate = d.gate_weights;
+  p.ffn1 = d.ffn1_weights;
+  p.ffn2 = d.ffn2_weights;
+  p.bias = d.router_bias;
+  p.out = output;
+  char* w = l->ws;
+  p.ctl = reinterpret_cast<fmoe::Control*>(w + L.ctl);
+  p.g1_done = reinterpret_cast<unsigned*>(w + L.g1_done);
+  p.masks = reinterpret_cast<unsigned long long*>(w + L.masks);
+  p.word_prefix = reinterpret_cast<int*>(w + L.word_prefix);
+  p.topk_idx = reinterpret_cast<int*>(w + L.topk_idx);
+  p.topk_w = reinterpret_cast<float*>(w + L.topk_w);
+  p.expert_count = reinterpret_cast<int*>(w + L.expert_count);
+  p.expert_offset = reinterpret_cast<int*>(w + L.expert_offset);
+  p.perm = reinterpret_cast<int*>(w + L.perm);
+  p.row_w = reinterpret_cast<float*>(w + L.row_w);
+  p.mtiles = reinterpret_cast<fmoe::TileDesc*>(w + L.mtiles);
+  p.h = w + L.h;
+  p.y = reinterpret_cast<float*>(w + L.y);
+  return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* flashMoeVersion(void) { return "flashMoe-mi355x 0.1 (gfx950)"; }
+
+int flashMoeWorkspaceBytes(const FlashMoeLayerDesc* desc, size_t* bytes) {
+  const hipError_t v = validate(desc);
+  if (v != hipSuccess) return v;
+  if (bytes == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null result pointer");
+  *bytes = make_layout(*desc).total;
+  return hipSuccess;
+}
+
+int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const hipError_t v = validate(desc);
+  if (v != hipSuccess) return v;
+  if (out == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher result pointer");
+  if (desc->gate_weights == nullptr || desc->ffn1_weights == nullptr ||
+      desc->ffn2_weights == nullptr)
+    FMOE_FAIL(hipErrorInvalidValue, "null weight pointer");
+
+  FlashMoeLauncher* l = new (std::nothrow) FlashMoeLauncher();
+  if (l == nullptr) FMOE_FAIL(hipErrorOutOfMemory, "host allocation failed");
+  l->desc = *desc;
+  l->layout = make_layout(*desc);
+
+  auto fail = [&](hipError_t e) {
+    if (l->ws) (void)hipFree(l->ws);
+    delete l;
+    printf("[MOE HIP ERROR: %s]: create failed: %s\n", FMOE_FILENAME, hipGetErrorString(e));
+    return static_cast<int>(e);
+  };
+  hipError_t e;
+  if ((e = hipGetDevice(&l->device)) != hipSuccess) return fail(e);
+  if ((e = hipDeviceGetAttribute(&l->num_cus, hipDeviceAttributeMultiprocessorCount,
+                                 l->device)) != hipSuccess)
+    return fail(e);
+  int khz = 0;
+  if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, l->device) == hipSuccess &&
+      khz > 0)
+    l->ticks_per_ms = khz;
+  l->spin_limit = 2000 * l->ticks_per_ms;
+  if ((e = hipMalloc(reinterpret_cast<void**>(&l->ws), l->layout.total)) != hipSuccess)
+    return fail(e);
+  if ((e = hipMemsetAsync(l->ws, 0, l->layout.zero_bytes, stream)) != hipSuccess) return fail(e);
+  if ((e = hipStreamSynchronize(stream)) != hipSuccess) return fail(e);
+  *out = l;
+  return hipSuccess;
+}
+
+int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num) {
+  (void)tokens_num;
+  if (l == nullptr) return -1;
+  return FLASH_MOE_SCHED_STREAM;
+}
+
+int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int tokens_num,
+                   void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (l == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher");
+  if (tokens_num < 0) FMOE_FAIL(hipErrorInvalidValue, "tokens_num = %i", tokens_num);
+  if (tokens_num > l->desc.max_tokens)
+    FMOE_FAIL(hipErrorUnknown, "tokens_num = %i exceeds max_tokens = %i", tokens_num,
+              l->desc.max_tokens);
+  if (tokens_num == 0) return hipSuccess;
+  if (tokens == nullptr || output == nullptr)
+    FMOE_FAIL(hipErrorInvalidValue, "null tokens/output pointer");
+  const fmoe::Params p = make_params(l, tokens, output, tokens_num);
+  l->last_tokens = tokens_num;
+  FMOE_HIP_CHECK(fmoe::launch_stream_kernel(p, l->desc.dtype, l->num_cus, stream));
+  return hipSuccess;
+}
+
+int flashMoeDestroy(FlashMoeLauncher* l, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (l == nullptr) return hipSuccess;
+  FMOE_HIP_CHECK(hipStreamSynchronize(stream));
+  FMOE_HIP_CHECK(hipFree(l->ws));
+  delete l;
+  return hipSuccess;
+}
+
+int flashMoeReadRouting(FlashMoeLauncher* l, int tokens_num, int* topk_idx, float* topk_w,
+                        int* expert_counts, int* expert_offsets, int* perm, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (l == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher");
+  if (tokens_num < 0 || tokens_num > l->desc.max_tokens)
+    FMOE_FAIL(hipErrorInvalidValue, "tokens_num = %i", tokens_num);
+  FMOE_HIP_CHECK(hipStreamSynchronize(stream));
+  const size_t rows = static_cast<size_t>(tokens_num) * l->desc.top_k;
+  const Layout& L = l->layout;
+  if (topk_idx)
+    FMOE_HIP_CHECK(hipMemcpy(topk_idx, l->ws + L.topk_idx, sizeof(int) * rows,
+                             hipMemcpyDeviceToHost));
+  if (topk_w)
+    FMOE_HIP_CHECK(hipMemcpy(topk_w, l->ws + L.topk_w, sizeof(float) * rows,
+                             hipMemcpyDeviceToHost));
+  if (expert_counts)
+    FMOE_HIP_CHECK(hipMemcpy(expert_counts, l->ws + L.expert_count, sizeof(int) * l->desc.experts,
+                             hipMemcpyDeviceToHost));
+  if (expert_offsets)
+    FMOE_HIP_CHECK(hipMemcpy(expert_offsets, l->ws + L.expert_offset,
+                             sizeof(int) * (l->desc.experts + 1), hipMemcpyDeviceToHost));
+  if (perm)
+    FMOE_HIP_CHECK(hipMemcpy(perm, l->ws + L.perm, sizeof(int) * rows, hipMemcpyDeviceToHost));
+  return hipSuccess;
+}
+
+int flashMoeStatus(FlashMoeLauncher* l, unsigned* error_bits, unsigned* launches, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (l == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher");
+  FMOE_HIP_CHECK(hipStreamSynchronize(stream));
+  fmoe::Control c;
+  FMOE_HIP_CHECK(hipMemcpy(&c, l->ws + l->layout.ctl, sizeof(c), hipMemcpyDeviceToHost));
+  if (error_bits) *error_bits = c.error;
+  if (launches) *launches = c.launches;
+  if (c.error != 0u) {
+    // an aborted launch leaves counters and masks in an arbitrary state
+    FMOE_HIP_CHECK(hipMemset(l->ws, 0, l->layout.zero_bytes));
+  }
+  return hipSuccess;
+}
+
+int flashMoeSetWaitLimitMs(FlashMoeLauncher* l, double ms) {
+  if (l == nullptr || !(ms > 0.0)) FMOE_FAIL(hipErrorInvalidValue, "bad wait limit");
+  l->spin_limit = static_cast<long long>(ms * static_cast<double>(l->ticks_per_ms));
+  if (l->spin_limit < 1) l->spin_limit = 1;
+  return hipSuccess;
+}
+
+}  // extern "C"
+
+// ------------------------------------------------- C++ interface (drop-in)
+namespace moe {
+
+IMoeKernelLauncher::~IMoeKernelLauncher() {}
+
+namespace {
+class FusedMoeLauncher final : public IMoeKernelLauncher {
+ public:
+  explicit FusedMoeLauncher(FlashMoeLauncher* h) : handle_(h) {}
+  hipError_t Launch(const void* tokens, void* output, int tokensNum,
+                    hipStream_t stream) override {
+    return static_cast<hipError_t>(flashMoeLaunch(handle_, tokens, output, tokensNum, stream));
+  }
+  FlashMoeLauncher* handle() const { return handle_; }
+  void release() { handle_ = nullptr; }
+
+ private:
+  FlashMoeLauncher* handle_;
+};
+}  // namespace
+}  // namespace moe
+
+extern "C" {
+
+moe::DistributedUniqueId GetDistributedUniqueId(bool empty) {
+  // The reference asks rocSHMEM for an id unless `empty`
+  // (src/moeKernelLauncher.cpp:15-30). There is no inter-GPU transport here,
+  // so both cases give the all-zero id.
+  (void)empty;
+  moe::DistributedUniqueId id;
+  memset(id.data, 0, sizeof(id.data));
+  return id;
+}
+
+hipError_t CreateLauncherEx(moe::IMoeKernelLauncher** launcher, const FlashMoeLayerDesc* desc,
+                            hipStream_t stream) {
+  if (launcher == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher result pointer");
+  FlashMoeLauncher* h = nullptr;
+  const int e = flashMoeCreate(&h, desc, stream);
+  if (e != hipSuccess) return static_cast<hipError_t>(e);
+  moe::FusedMoeLauncher* obj = new (std::nothrow) moe::FusedMoeLauncher(h);
+  if (obj == nullptr) {
+    (void)flashMoeDestroy(h, stream);
+    FMOE_FAIL(hipErrorOutOfMemory, "host allocation failed");
+  }
+  *launcher = obj;
+  return hipSuccess;
+}
+
+hipError_t CreateLauncher(moe::IMoeKernelLauncher** launcher, const void* gateWeights,
+                          const void* ffn1ExpertWeights, const void* ffn2ExpertWeights,
+                          int maxTokens, hipStream_t stream, const moe::DistributedUniqueId& uid,
+                          int rank, int worldSize) {
+  (void)uid;
+  // shape of src/hip/common/metadata.h:7-13
+  FlashMoeLayerDesc d{};
+  d.experts = 128;
+  d.hidden = 2048;
+  d.intermediate = 768;
+  d.top_k = 8;
+  d.dtype = FLASH_MOE_F32;
+  d.max_tokens = maxTokens;
+  d.sched = FLASH_MOE_SCHED_AUTO;
+  d.gate_weights = gateWeights;
+  d.ffn1_weights = ffn1ExpertWeights;
+  d.ffn2_weights = ffn2ExpertWeights;
+  d.router_bias = nullptr;
+  if (worldSize != 1 || rank != 0)
+    FMOE_FAIL(hipErrorInvalidValue,
+              "rank %i of %i: only rank 0 of a world of 1 is supported (no inter-GPU transport)",
+              rank, worldSize);
+  return CreateLauncherEx(launcher, &d, stream);
+}
+
+hipError_t DestroyLauncher(moe::IMoeKernelLauncher* launcher, hipStream_t stream) {
+  if (launcher == nullptr) return hipSuccess;
+  moe::FusedMoeLauncher* obj = static_cast<moe::FusedMoeLauncher*>(launcher);
+  const int e = flashMoeDestroy(obj->handle(), stream);
+  if (e != hipSuccess) return static_cast<hipError_t>(e);
+  delete obj;
+  return hipSuccess;
+}
+
+FlashMoeLauncher* LauncherHandle(moe::IMoeKernelLauncher* launcher) {
+  if (launcher == nullptr) return nullptr;
+  return static_cast<moe::FusedMoeLauncher*>(launcher)->handle();
+}
+
+}  // extern "C"

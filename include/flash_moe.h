@@ -1,0 +1,105 @@
+/* C ABI of the MI355X fused MoE layer (libflashMoe.so).
+ *
+ * Plain pointers and sizes only; every pointer named "device" is HBM owned by
+ * the caller. This is the layer the C++ interface in iMoeKernelLauncher.h and
+ * any foreign-function binding (ctypes, cgo, JNI ...) sit on. All functions
+ * return a hipError_t value as int (0 = hipSuccess) and never throw.
+ *
+ * What each entry point replaces in the reference (paths relative to the
+ * reference checkout):
+ *   flashMoeCreate      CreateLauncher  -> MoeKernelLauncher::Init
+ *                       (src/moeKernelLauncher.cpp:33-46,
+ *                        src/hip/launcher/moeKernelLauncher.hip:96-187), with the
+ *                       compile-time shape of src/hip/common/metadata.h:7-13
+ *                       turned into run-time fields
+ *   flashMoeLaunch      IMoeKernelLauncher::Launch
+ *                       (include/iMoeKernelLauncher.h:12-13,
+ *                        src/hip/launcher/moeKernelLauncher.hip:58-93,207-212)
+ *   flashMoeDestroy     DestroyLauncher -> MoeKernelLauncher::Deinit
+ *                       (src/moeKernelLauncher.cpp:49-55,
+ *                        src/hip/launcher/moeKernelLauncher.hip:190-204)
+ *   flashMoeReadRouting no counterpart: copies the router's decisions out so
+ *                       that tests can compare them bit for bit, as the
+ *                       reference's stage test does for its gate
+ *                       (test/singleGPU/cpp/moe/internal/moeGateTest.hip:62-109)
+ *   flashMoeStatus      no counterpart: the reference asserts on the device
+ *                       (src/hip/utils/hipDeviceUtils.h:12); here a bounded wait
+ *                       that runs out raises a flag the host can read
+ */
+#ifndef FLASH_MOE_H_
+#define FLASH_MOE_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct FlashMoeLauncher FlashMoeLauncher; /* opaque */
+
+enum { FLASH_MOE_F32 = 0, FLASH_MOE_BF16 = 1 };
+
+/* Scheduling variant. AUTO picks by rows per expert. */
+enum { FLASH_MOE_SCHED_AUTO = 0, FLASH_MOE_SCHED_STREAM = 1, FLASH_MOE_SCHED_TILED = 2 };
+
+typedef struct FlashMoeLayerDesc {
+  int experts;      /* E, 1..256 */
+  int hidden;       /* H, multiple of 64 */
+  int intermediate; /* I, multiple of 32 */
+  int top_k;        /* k, 1..min(E,32) */
+  int dtype;        /* FLASH_MOE_F32 or FLASH_MOE_BF16: weights, tokens, output */
+  int max_tokens;   /* largest tokens_num a launch may pass */
+  int sched;        /* FLASH_MOE_SCHED_* */
+  int reserved;
+  const void* gate_weights;  /* device, [E,H] row-major */
+  const void* ffn1_weights;  /* device, [E,2I,H]: rows 0..I-1 gate proj, I..2I-1 up proj */
+  const void* ffn2_weights;  /* device, [E,H,I] */
+  const float* router_bias;  /* device, [E] float added to the logits, or NULL */
+} FlashMoeLayerDesc;
+
+/* Device bytes flashMoeCreate would allocate for this description. */
+int flashMoeWorkspaceBytes(const FlashMoeLayerDesc* desc, size_t* bytes);
+
+/* Allocates the workspace on the current device and synchronises `stream`.
+ * Weights are borrowed and must outlive the launcher. On failure *out is left
+ * untouched. hipErrorUnknown: max_tokens beyond capacity;
+ * hipErrorInvalidValue: anything else wrong with the description. */
+int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* stream);
+
+/* Enqueues one forward pass on `stream` and returns without waiting.
+ * tokens, output: device [tokens_num, H] in the layer dtype; output may alias
+ * tokens. Launches on one launcher must be ordered on one stream.
+ * hipErrorUnknown when tokens_num > max_tokens. */
+int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int tokens_num,
+                   void* stream);
+
+/* Frees the workspace; synchronises `stream`. */
+int flashMoeDestroy(FlashMoeLauncher* l, void* stream);
+
+/* After a launch of tokens_num tokens: waits for `stream`, then copies the
+ * routing of that launch to host arrays (any may be NULL):
+ * topk_idx [T,k], topk_w [T,k], expert_counts [E], expert_offsets [E+1],
+ * perm [T*k] (permuted row -> t*k+slot; only the first expert_offsets[E] are
+ * meaningful). */
+int flashMoeReadRouting(FlashMoeLauncher* l, int tokens_num, int* topk_idx, float* topk_w,
+                        int* expert_counts, int* expert_offsets, int* perm, void* stream);
+
+/* Waits for `stream`, reports the device error bits (1 = a dependency wait
+ * timed out, 2 = tile table overflow) and the number of completed launches.
+ * If error bits are set the launcher's counters are cleared so that it can be
+ * used again. */
+int flashMoeStatus(FlashMoeLauncher* l, unsigned* error_bits, unsigned* launches, void* stream);
+
+/* Bound on a single dependency wait inside the kernel, in milliseconds
+ * (default 2000). A wait that runs out raises error bit 1 and ends the launch. */
+int flashMoeSetWaitLimitMs(FlashMoeLauncher* l, double ms);
+
+/* Which scheduling variant a launch of tokens_num tokens would use. */
+int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num);
+
+const char* flashMoeVersion(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_MOE_H_ */
