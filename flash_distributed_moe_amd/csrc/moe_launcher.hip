@@ -21,6 +21,7 @@
 
 namespace fmoe {
 hipError_t launch_stream_kernel(const Params& p, int dtype, int grid, hipStream_t stream);
+hipError_t prepare_stream_kernel();
 }
 
 #define FMOE_FILENAME (strrchr(__FILE__, '/') ? strrchr(__FILE__, '/') + 1 : __FILE__)
@@ -50,11 +51,13 @@ constexpr long long kMaxRows = 1ll << 21;  // max_tokens * top_k a launcher may 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct Layout {
-  size_t ctl, g1_done, topk_idx, topk_w, masks, word_prefix, expert_count, expert_offset, perm,
-      row_w, mtiles, h, y, total;
+  size_t ctl, wgflags, g1_done, tok_arrive, cand, topk_idx, topk_w, masks, word_prefix,
+      expert_count, expert_offset, perm, row_w, mtiles, h, y, total;
   size_t zero_bytes;  // leading region that must be zero before a launch
   int W, max_mtiles;
 };
+
+constexpr int kMaxGroups = 1024;  // workgroups a launch may use (one per CU)
 
 Layout make_layout(const FlashMoeLayerDesc& d) {
   Layout L{};
@@ -70,9 +73,12 @@ Layout make_layout(const FlashMoeLayerDesc& d) {
   };
   // zero-initialised region first: control block, per-tile counters, masks
   L.ctl = take(sizeof(fmoe::Control));
-  L.g1_done = take(sizeof(unsigned) * L.max_mtiles);
+  L.wgflags = take(sizeof(fmoe::WgFlags) * kMaxGroups);
+  L.g1_done = take(sizeof(fmoe::ControlLine) * L.max_mtiles);
   L.masks = take(sizeof(unsigned long long) * d.experts * L.W);
+  L.tok_arrive = take(sizeof(unsigned) * d.max_tokens);
   L.zero_bytes = off;
+  L.cand = take(sizeof(unsigned long long) * d.max_tokens * d.experts);
   L.word_prefix = take(sizeof(int) * d.experts * L.W);
   L.topk_idx = take(sizeof(int) * rows);
   L.topk_w = take(sizeof(float) * rows);
@@ -126,6 +132,8 @@ struct FlashMoeLauncher {
   long long ticks_per_ms = 100000;
   long long spin_limit = 0;
   int last_tokens = 0;
+  fmoe::TraceRec* trace = nullptr;
+  unsigned trace_cap = 0;
 };
 
 namespace {
@@ -140,7 +148,9 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.K = d.top_k;
   p.I = d.intermediate;
   p.W = L.W;
-  p.n_workers = l->num_cus * 8;
+  p.n_groups = l->num_cus < kMaxGroups ? l->num_cus : kMaxGroups;
+  p.n_workers = p.n_groups * 8;
+  p.fuse_scatter = (static_cast<long long>(T) * d.top_k <= 2048) ? 1 : 0;
   p.max_mtiles = L.max_mtiles;
   p.spin_limit = l->spin_limit;
   p.tokens = tokens;
@@ -151,7 +161,10 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.out = output;
   char* w = l->ws;
   p.ctl = reinterpret_cast<fmoe::Control*>(w + L.ctl);
-  p.g1_done = reinterpret_cast<unsigned*>(w + L.g1_done);
+  p.wgflags = reinterpret_cast<fmoe::WgFlags*>(w + L.wgflags);
+  p.g1_done = reinterpret_cast<fmoe::ControlLine*>(w + L.g1_done);
+  p.tok_arrive = reinterpret_cast<unsigned*>(w + L.tok_arrive);
+  p.cand = reinterpret_cast<unsigned long long*>(w + L.cand);
   p.masks = reinterpret_cast<unsigned long long*>(w + L.masks);
   p.word_prefix = reinterpret_cast<int*>(w + L.word_prefix);
   p.topk_idx = reinterpret_cast<int*>(w + L.topk_idx);
@@ -163,6 +176,8 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.mtiles = reinterpret_cast<fmoe::TileDesc*>(w + L.mtiles);
   p.h = w + L.h;
   p.y = reinterpret_cast<float*>(w + L.y);
+  p.trace = l->trace;
+  p.trace_cap = l->trace_cap;
   return p;
 }
 
@@ -210,6 +225,8 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
       khz > 0)
     l->ticks_per_ms = khz;
   l->spin_limit = 2000 * l->ticks_per_ms;
+  if ((e = fmoe::prepare_stream_kernel()) != hipSuccess)
+    return fail(e);
   if ((e = hipMalloc(reinterpret_cast<void**>(&l->ws), l->layout.total)) != hipSuccess)
     return fail(e);
   if ((e = hipMemsetAsync(l->ws, 0, l->layout.zero_bytes, stream)) != hipSuccess) return fail(e);
@@ -237,7 +254,7 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
     FMOE_FAIL(hipErrorInvalidValue, "null tokens/output pointer");
   const fmoe::Params p = make_params(l, tokens, output, tokens_num);
   l->last_tokens = tokens_num;
-  FMOE_HIP_CHECK(fmoe::launch_stream_kernel(p, l->desc.dtype, l->num_cus, stream));
+  FMOE_HIP_CHECK(fmoe::launch_stream_kernel(p, l->desc.dtype, p.n_groups, stream));
   return hipSuccess;
 }
 
@@ -246,6 +263,7 @@ int flashMoeDestroy(FlashMoeLauncher* l, void* stream_) {
   if (l == nullptr) return hipSuccess;
   FMOE_HIP_CHECK(hipStreamSynchronize(stream));
   FMOE_HIP_CHECK(hipFree(l->ws));
+  if (l->trace) FMOE_HIP_CHECK(hipFree(l->trace));
   delete l;
   return hipSuccess;
 }
@@ -282,12 +300,40 @@ int flashMoeStatus(FlashMoeLauncher* l, unsigned* error_bits, unsigned* launches
   FMOE_HIP_CHECK(hipStreamSynchronize(stream));
   fmoe::Control c;
   FMOE_HIP_CHECK(hipMemcpy(&c, l->ws + l->layout.ctl, sizeof(c), hipMemcpyDeviceToHost));
-  if (error_bits) *error_bits = c.error;
-  if (launches) *launches = c.launches;
-  if (c.error != 0u) {
+  if (error_bits) *error_bits = c.error.v;
+  if (launches) *launches = c.launches.v;
+  if (c.error.v != 0u) {
     // an aborted launch leaves counters and masks in an arbitrary state
     FMOE_HIP_CHECK(hipMemset(l->ws, 0, l->layout.zero_bytes));
   }
+  return hipSuccess;
+}
+
+int flashMoeTraceEnable(FlashMoeLauncher* l, unsigned capacity) {
+  if (l == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher");
+  FMOE_HIP_CHECK(hipDeviceSynchronize());
+  if (l->trace) {
+    FMOE_HIP_CHECK(hipFree(l->trace));
+    l->trace = nullptr;
+    l->trace_cap = 0;
+  }
+  if (capacity == 0) return hipSuccess;
+  FMOE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&l->trace),
+                           sizeof(fmoe::TraceRec) * static_cast<size_t>(capacity)));
+  FMOE_HIP_CHECK(hipMemset(l->trace, 0xFF, sizeof(fmoe::TraceRec) * static_cast<size_t>(capacity)));
+  l->trace_cap = capacity;
+  return hipSuccess;
+}
+
+int flashMoeTraceRead(FlashMoeLauncher* l, void* records, unsigned max_records, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (l == nullptr || records == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null argument");
+  if (l->trace == nullptr) FMOE_FAIL(hipErrorInvalidValue, "tracing is not enabled");
+  FMOE_HIP_CHECK(hipStreamSynchronize(stream));
+  const unsigned n = max_records < l->trace_cap ? max_records : l->trace_cap;
+  FMOE_HIP_CHECK(hipMemcpy(records, l->trace, sizeof(fmoe::TraceRec) * static_cast<size_t>(n),
+                           hipMemcpyDeviceToHost));
+  FMOE_HIP_CHECK(hipMemset(l->trace, 0xFF, sizeof(fmoe::TraceRec) * static_cast<size_t>(l->trace_cap)));
   return hipSuccess;
 }
 

@@ -25,20 +25,31 @@ constexpr int COMBINE_COLS = 256;
 constexpr int MAX_EXPERTS = 256;  // experts are spread 64 per wave register slot
 constexpr int MAX_TOPK = 32;
 
-// Dependency counters and the ticket dispenser. Everything up to `error` is
-// zero before a launch and is returned to zero by the last worker to leave.
+// Dependency counters and the ticket dispenser, one 128-byte line each so that
+// pollers of one counter do not queue behind atomics on another. Everything
+// except `error` and `launches` is zero before a launch and is returned to zero
+// by the last worker to leave.
+struct alignas(128) ControlLine {
+  unsigned v;
+  unsigned pad[31];
+};
 struct Control {
-  unsigned ticket;       // next task number
-  unsigned router_done;  // router tasks finished
-  unsigned scan_done;    // 1 once expert offsets and the tile table exist
-  unsigned perm_done;    // scatter tasks finished
-  unsigned g2_done;      // down-projection tasks finished
-  unsigned exit_count;   // workers that have left the loop
-  unsigned n_mtiles;     // row tiles produced by the scan
-  unsigned reserved0;
-  unsigned error;        // sticky error bits
-  unsigned launches;     // completed launches (diagnostic)
-  unsigned reserved1[6];
+  ControlLine ticket;       // next task number
+  ControlLine router_done;  // tokens whose routing is final
+  ControlLine perm_done;    // scatter tasks finished
+  ControlLine g2_done;      // down-projection tasks finished
+  ControlLine exit_count;   // workers that have left the loop
+  ControlLine n_mtiles;     // row tiles produced by the scan
+  ControlLine error;        // sticky error bits
+  ControlLine launches;     // completed launches (diagnostic)
+};
+
+// Phase flags, one line per workgroup: the worker that completes a phase
+// writes every workgroup's copy, so waiting workers poll a line nobody else
+// touches instead of queueing on one address.
+enum : int { FLAG_SCAN = 0, FLAG_PERM = 1, FLAG_G2 = 2 };
+struct alignas(128) WgFlags {
+  unsigned f[32];
 };
 
 struct TileDesc {  // one row tile: `rows` consecutive permuted rows of one expert
@@ -46,6 +57,18 @@ struct TileDesc {  // one row tile: `rows` consecutive permuted rows of one expe
   int row0;
   int rows;
   int pad;
+};
+
+// One record per executed task when tracing is on (times: 100 MHz wall clock).
+struct TraceRec {
+  unsigned ticket;
+  unsigned kind;    // 0 router dot, 1 scan, 2 scatter, 3 gate/up, 4 down, 5 combine, 6 select
+  unsigned worker;  // workgroup * waves_per_group + wave
+  unsigned aux;     // task-specific (row tile, token ...)
+  long long t_fetch;  // before the ticket was drawn
+  long long t_ready;  // dependencies satisfied, work starts
+  long long t_end;    // work finished and signalled
+  long long pad;
 };
 
 struct Params {
@@ -74,7 +97,14 @@ struct Params {
   void* h;                    // [T*K, I] SwiGLU output, layer dtype
   float* y;                   // [T*K, H] weighted down-projection rows, by t*K+slot
   Control* ctl;
-  unsigned* g1_done;  // [max_mtiles] gate/up tasks finished per row tile
+  WgFlags* wgflags;                // [n_groups]
+  ControlLine* g1_done;            // [max_mtiles] gate/up tasks finished per row tile
+  unsigned long long* cand;        // [T,E] router candidate keys
+  unsigned* tok_arrive;            // [T] expert groups of the token whose keys are in
+  int n_groups;                    // workgroups in the grid
+  int fuse_scatter;                // 1: the scan task also writes the permutation
+  TraceRec* trace;    // null unless tracing; indexed by ticket
+  unsigned trace_cap;
 };
 
 }  // namespace fmoe

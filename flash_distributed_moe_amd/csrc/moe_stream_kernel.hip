@@ -14,6 +14,8 @@
 //   combine  (token, 256 columns): out = sum over slots of y, in slot order
 // Weights stream HBM -> registers -> MFMA with no reuse across waves, which is
 // the right shape when an expert sees at most a few dozen rows (decode).
+// The down projection reads h rows that other workers wrote, so its B operand
+// uses the coherent loads described below.
 //
 // Replaces, for this regime, the reference's moeKernel
 // (src/hip/kernel/moeKernel.h:37-107), its task executors
@@ -38,25 +40,114 @@ struct BF16 {
 };
 
 // ------------------------------------------------------------------ helpers
+// Coherence between workers. MI355X has eight XCDs with one L2 each, and an
+// agent-scope release/acquire fence writes back / invalidates a whole L2: with
+// two thousand waves signalling, each fence costs tens of microseconds. So
+// nothing here uses those fences. Every value one worker produces for another
+// (routing tables, h, y, counters) is written and read with agent-scope relaxed
+// atomic accesses of 4 or 8 bytes, which go through to the memory-side
+// coherence point; a producer waits for its stores (workgroup-scope release =
+// wait for outstanding memory operations) and then bumps a counter, a consumer
+// polls the counter and then loads. Inputs (tokens, weights) are never written
+// while the kernel runs and use ordinary cached loads.
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 
-__device__ __forceinline__ unsigned ld_relaxed(const unsigned* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void fence_acquire() {
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-}
-__device__ __forceinline__ void fence_release() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-}
-__device__ __forceinline__ unsigned add_relaxed(unsigned* p, unsigned v) {
-  return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Every pointer in Params is HBM: saying so lets the compiler emit global_*
+// instead of flat_* memory instructions (flat ones also count as LDS traffic).
+#define FMOE_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ FMOE_GLOBAL T* as_global(T* p) {
+  return (FMOE_GLOBAL T*)p;
 }
 
-// All lanes' earlier stores become visible device-wide, then the counter moves.
-__device__ __forceinline__ void wave_signal(unsigned* counter) {
+__device__ __forceinline__ unsigned ldc(const unsigned* p) {
+  return __hip_atomic_load(as_global(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int ldc(const int* p) {
+  return __hip_atomic_load(as_global(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ldc(const float* p) {
+  return __uint_as_float(__hip_atomic_load(as_global(reinterpret_cast<const unsigned*>(p)),
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+__device__ __forceinline__ unsigned long long ldc(const unsigned long long* p) {
+  return __hip_atomic_load(as_global(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void stc(unsigned* p, unsigned v) {
+  __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void stc(int* p, int v) {
+  __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void stc(float* p, float v) {
+  __hip_atomic_store(as_global(reinterpret_cast<unsigned*>(p)), __float_as_uint(v),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void stc(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// 16 coherent bytes as two 8-byte accesses
+__device__ __forceinline__ uint4 ldc16(const void* p) {
+  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
+  const unsigned long long a = ldc(q), b = ldc(q + 1);
+  return make_uint4(static_cast<unsigned>(a), static_cast<unsigned>(a >> 32),
+                    static_cast<unsigned>(b), static_cast<unsigned>(b >> 32));
+}
+__device__ __forceinline__ void stc16(void* p, const uint4& v) {
+  unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+  stc(q, static_cast<unsigned long long>(v.x) | (static_cast<unsigned long long>(v.y) << 32));
+  stc(q + 1, static_cast<unsigned long long>(v.z) | (static_cast<unsigned long long>(v.w) << 32));
+}
+__device__ __forceinline__ TileDesc ld_tile(const TileDesc* t) {
+  const uint4 v = ldc16(t);
+  TileDesc d;
+  d.expert = static_cast<int>(v.x);
+  d.row0 = static_cast<int>(v.y);
+  d.rows = static_cast<int>(v.z);
+  d.pad = 0;
+  return d;
+}
+
+__device__ __forceinline__ unsigned ld_relaxed(const unsigned* p) {
+  return __hip_atomic_load(as_global(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Ordering only (no cache maintenance): later loads stay after the poll that
+// precedes this / earlier stores have completed before the counter moves.
+__device__ __forceinline__ void fence_acquire() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+__device__ __forceinline__ void fence_release() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);  // every outstanding store has reached the coherence point
+}
+__device__ __forceinline__ unsigned add_relaxed(unsigned* p, unsigned v) {
+  return __hip_atomic_fetch_add(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_relaxed(unsigned* p, unsigned v) {
+  __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void or_relaxed(unsigned* p, unsigned v) {
+  __hip_atomic_fetch_or(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void or_relaxed(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_fetch_or(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// All lanes' earlier coherent stores have completed, then the counter moves.
+// Returns the counter's previous value to every lane.
+__device__ __forceinline__ unsigned wave_arrive(unsigned* counter) {
   fence_release();
-  if (lane_id() == 0) add_relaxed(counter, 1u);
+  unsigned old = 0;
+  if (lane_id() == 0) old = add_relaxed(counter, 1u);
+  return __builtin_amdgcn_readfirstlane(old);
+}
+
+// Called by the worker that completed a phase (after wave_arrive told it so, or
+// after its own release fence): raises the phase flag of every workgroup.
+__device__ __forceinline__ void broadcast_flag(const Params& p, int which) {
+  const int n = p.n_groups;
+  WgFlags* flags = p.wgflags;
+  for (int g = lane_id(); g < n; g += 64) st_relaxed(&flags[g].f[which], 1u);
 }
 
 // Wave-uniform bounded wait for *p >= target. False on time-out or when
@@ -67,18 +158,18 @@ __device__ __forceinline__ bool wave_wait_ge(const unsigned* p, unsigned target,
   if (lane_id() == 0) {
     if (ld_relaxed(p) < target) {
       const long long t0 = wall_clock64();
+      unsigned spins = 0;
       while (ld_relaxed(p) < target) {
-        if (ld_relaxed(&ctl->error) != 0u) {
+        if ((++spins & 31u) == 0u && ld_relaxed(&ctl->error.v) != 0u) {
           ok = 0;
           break;
         }
         if (wall_clock64() - t0 > limit) {
-          __hip_atomic_fetch_or(&ctl->error, ERR_TIMEOUT, __ATOMIC_RELAXED,
-                                __HIP_MEMORY_SCOPE_AGENT);
+          or_relaxed(&ctl->error.v, ERR_TIMEOUT);
           ok = 0;
           break;
         }
-        __builtin_amdgcn_s_sleep(8);
+        __builtin_amdgcn_s_sleep(16);
       }
     }
   }
@@ -87,8 +178,13 @@ __device__ __forceinline__ bool wave_wait_ge(const unsigned* p, unsigned target,
   return ok != 0;
 }
 
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 ld16(const void* p) {
-  return *reinterpret_cast<const uint4*>(p);
+  const u32x4 v = *as_global(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st16(void* p, const u32x4& v) {
+  *as_global(reinterpret_cast<u32x4*>(p)) = v;
 }
 
 __device__ __forceinline__ float bf16_lo(unsigned u) { return __uint_as_float(u << 16); }
@@ -169,131 +265,326 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
 // (refTopk.h:36-58), weights are a softmax over the winners in double
 // (refMoeGate.h:27-30, refSoftmax.h:19-52). For bf16 inputs each product is
 // exact in float, so the fused multiply-add below rounds exactly as mul+add.
-template <typename DT>
-__device__ void router_task(const Params& p, int t) {
-  typedef typename DT::elem elem;
-  constexpr int EPV = DT::EPV;
+//
+// The logits are computed by "dot" tasks: one wave takes 8 tokens x 8 experts,
+// one (token, expert) chain per lane. Token rows and expert rows arrive with
+// fully coalesced 16-byte loads, are converted to float once and staged in the
+// wave's private LDS slice in k-chunks, and feed one sequential chain per lane
+// (k ascending). Each chain ends as a 64-bit candidate key in HBM. A "select"
+// task per token waits for all of the token's expert groups and picks the
+// winners.
+constexpr int ROUTER_TOK = 8;    // tokens per dot task
+constexpr int ROUTER_EXP = 8;    // experts per dot task
+constexpr int ROUTER_KC = 256;   // k-chunk staged in LDS
+constexpr int ROUTER_LD = ROUTER_KC + 4;  // LDS row stride in floats (bank spread)
+constexpr int ROUTER_LDS_FLOATS = 2 * ROUTER_EXP * ROUTER_LD;  // per wave
+
+// (order-preserving value bits, inverted index): the maximum key is the largest
+// value and, among equals, the lowest index. Values the reference's strict '>'
+// against lowest() never admits (NaN, -inf, -FLT_MAX) get key 0.
+__device__ __forceinline__ unsigned long long make_key(float v, int e, bool in_range) {
+  const bool valid = in_range && (v > -FLT_MAX);
+  unsigned u = __float_as_uint(v);
+  u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  return valid ? ((static_cast<unsigned long long>(u) << 32) |
+                  static_cast<unsigned long long>(0xFFFFFFFFu - static_cast<unsigned>(e)))
+               : 0ull;
+}
+
+extern __shared__ __align__(16) float lds_dyn[];  // ROUTER_LDS_FLOATS per wave
+
+// Orders this wave's LDS writes before its later LDS reads (other lanes' data)
+// without waiting for global loads that are still in flight.
+__device__ __forceinline__ void lds_wave_sync() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// key[j] belongs to expert lane + 64*j. Writes the token's routing. Keys are
+// distinct (the index is part of the key), so a key's rank — how many keys are
+// greater — is its slot; ranks come from one pass over all keys in LDS.
+__device__ void router_select(const Params& p, int t, unsigned long long (&key)[MAX_EXPERTS / 64]) {
   constexpr int MAXEPL = MAX_EXPERTS / 64;
   const int lane = lane_id();
-  const int epl = (p.E + 63) >> 6;
-
-  const elem* x = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(t) * p.H;
-  const elem* wrow[MAXEPL];
-  float acc[MAXEPL];
+  const int E = p.E, K = p.K;
+  unsigned long long* lk =
+      reinterpret_cast<unsigned long long*>(lds_dyn + (threadIdx.x >> 6) * ROUTER_LDS_FLOATS);
+  unsigned long long* win = lk + MAX_EXPERTS;              // [MAX_TOPK] winning keys by slot
+  double* lex = reinterpret_cast<double*>(win + MAX_TOPK);  // [MAX_TOPK] exp terms
+  const int epl = (E + 63) >> 6;
 #pragma unroll
-  for (int j = 0; j < MAXEPL; ++j) {
-    int e = lane + 64 * j;
-    e = e < p.E ? e : p.E - 1;
-    wrow[j] = reinterpret_cast<const elem*>(p.gate) + static_cast<size_t>(e) * p.H;
-    acc[j] = 0.0f;
+  for (int j = 0; j < MAXEPL; ++j)
+    if (j < epl) lk[lane + 64 * j] = key[j];
+  if (lane < MAX_TOPK) win[lane] = 0ull;
+  lds_wave_sync();
+  int rank[MAXEPL];
+#pragma unroll
+  for (int j = 0; j < MAXEPL; ++j) rank[j] = 0;
+  const int n = epl * 64;
+  for (int i = 0; i < n; i += 2) {
+    const ulonglong2 o = *reinterpret_cast<const ulonglong2*>(lk + i);
+#pragma unroll
+    for (int j = 0; j < MAXEPL; ++j) rank[j] += (o.x > key[j] ? 1 : 0) + (o.y > key[j] ? 1 : 0);
   }
+#pragma unroll
+  for (int j = 0; j < MAXEPL; ++j)
+    if (j < epl && key[j] != 0ull && rank[j] < K) win[rank[j]] = key[j];
+  lds_wave_sync();
 
-#pragma unroll 2
-  for (int k0 = 0; k0 < p.H; k0 += EPV) {
-    float xf[EPV];
-    unpack<DT>(ld16(x + k0), xf);
+  int my_idx = -1;
+  float my_val = -FLT_MAX;
+  if (lane < K) {
+    const unsigned long long k64 = win[lane];
+    if (k64 != 0ull) {
+      my_idx = static_cast<int>(0xFFFFFFFFu - static_cast<unsigned>(k64 & 0xFFFFFFFFull));
+      unsigned u = static_cast<unsigned>(k64 >> 32);
+      u = (u & 0x80000000u) ? (u & 0x7FFFFFFFu) : ~u;
+      my_val = __uint_as_float(u);
+    }
+  }
+  // softmax over the K winners (descending, so the first is the maximum)
+  const unsigned long long k0 = win[0];
+  float v0f = -FLT_MAX;
+  if (k0 != 0ull) {
+    unsigned u = static_cast<unsigned>(k0 >> 32);
+    u = (u & 0x80000000u) ? (u & 0x7FFFFFFFu) : ~u;
+    v0f = __uint_as_float(u);
+  }
+  const double ex = lane < K ? exp(static_cast<double>(my_val) - static_cast<double>(v0f)) : 0.0;
+  if (lane < K) lex[lane] = ex;
+  lds_wave_sync();
+  double sum = 0.0;
+  for (int s = 0; s < K; ++s) sum += lex[s];
+  if (lane < K) {
+    const float w = sum <= 0.0 ? static_cast<float>(1.0 / static_cast<double>(K))
+                               : static_cast<float>(ex / sum);
+    stc(&p.topk_idx[static_cast<size_t>(t) * K + lane], my_idx);
+    stc(&p.topk_w[static_cast<size_t>(t) * K + lane], w);
+    if (my_idx >= 0) {
+      or_relaxed(&p.masks[static_cast<size_t>(my_idx) * p.W + (t >> 6)], 1ull << (t & 63));
+    }
+  }
+  lds_wave_sync();
+}
+
+template <typename DT>
+__device__ __noinline__ void router_dot_task(const Params& p, int tg, int eg) {
+  typedef typename DT::elem elem;
+  constexpr int EPV = DT::EPV;
+  constexpr int CH_ROW = ROUTER_KC / EPV;               // 16-byte chunks per staged row
+  constexpr int NLD = ROUTER_EXP * CH_ROW / 64;         // loads per lane per tile and chunk
+  // Params is reached through a generic reference; keep what the loops need in
+  // registers so that LDS stores do not force reloads.
+  const int H = p.H, E = p.E, T = p.T;
+  const int lane = lane_id();
+  const int ti = lane >> 3, ei = lane & 7;
+  const int t = tg * ROUTER_TOK + ti;
+  const int e = eg * ROUTER_EXP + ei;
+  float* ws = lds_dyn + (threadIdx.x >> 6) * ROUTER_LDS_FLOATS;  // [ROUTER_EXP][ROUTER_LD]
+  float* xs = ws + ROUTER_EXP * ROUTER_LD;                       // [ROUTER_TOK][ROUTER_LD]
+  const elem* gate = reinterpret_cast<const elem*>(p.gate);
+  const elem* tokens = reinterpret_cast<const elem*>(p.tokens);
+
+  // PF k-chunks of global loads are in flight ahead of the chunk being consumed
+#ifndef FMOE_ROUTER_PF
+#define FMOE_ROUTER_PF 1
+#endif
+  constexpr int PF = EPV == 8 ? FMOE_ROUTER_PF : (FMOE_ROUTER_PF + 1) / 2;
+  uint4 wr[PF][NLD], xr[PF][NLD];
+  auto issue = [&](uint4(&wq)[NLD], uint4(&xq)[NLD], int c0) {  // global -> registers
+    if (c0 >= H) return;
+    const int ch_row = min(ROUTER_KC, H - c0) / EPV;
 #pragma unroll
-    for (int j = 0; j < MAXEPL; ++j) {
-      if (j < epl) {
-        float wf[EPV];
-        unpack<DT>(ld16(wrow[j] + k0), wf);
+    for (int i = 0; i < NLD; ++i) {
+      // no branches around the loads: rows past the tile (short last chunk)
+      // re-read the last row and are dropped when staging
+      const int c = i * 64 + lane;
+      const int row = min(c / ch_row, ROUTER_EXP - 1), col = c % ch_row;
+      const int er = min(eg * ROUTER_EXP + row, E - 1);
+      const int tr = min(tg * ROUTER_TOK + row, T - 1);
+      wq[i] = ld16(gate + static_cast<size_t>(er) * H + c0 + col * EPV);
+      xq[i] = ld16(tokens + static_cast<size_t>(tr) * H + c0 + col * EPV);
+    }
+  };
+  auto stage = [&](const uint4(&wq)[NLD], const uint4(&xq)[NLD], int n) {  // -> float rows in LDS
+    const int ch_row = n / EPV;
 #pragma unroll
-        for (int i = 0; i < EPV; ++i) {
-          if constexpr (EPV == 8) {
-            acc[j] = __builtin_fmaf(xf[i], wf[i], acc[j]);
-          } else {
-            acc[j] = __fadd_rn(acc[j], __fmul_rn(xf[i], wf[i]));
-          }
+    for (int i = 0; i < NLD; ++i) {
+      const int c = i * 64 + lane;
+      const int row = c / ch_row, col = c % ch_row;
+      if (row < ROUTER_EXP) {
+        float wf[EPV], xf[EPV];
+        unpack<DT>(wq[i], wf);
+        unpack<DT>(xq[i], xf);
+#pragma unroll
+        for (int q = 0; q < EPV; q += 4) {
+          *reinterpret_cast<float4*>(ws + row * ROUTER_LD + col * EPV + q) =
+              make_float4(wf[q], wf[q + 1], wf[q + 2], wf[q + 3]);
+          *reinterpret_cast<float4*>(xs + row * ROUTER_LD + col * EPV + q) =
+              make_float4(xf[q], xf[q + 1], xf[q + 2], xf[q + 3]);
         }
+      }
+    }
+  };
+
+  float acc = 0.0f;
+  const float* wrow = ws + ei * ROUTER_LD;
+  const float* xrow = xs + ti * ROUTER_LD;
+  auto consume = [&](int n) {
+    // 32 k per block; the next block's LDS reads are in flight while this
+    // block's chain runs (n is a multiple of 64)
+    float4 wa[8], xa[8], wb[8], xb[8];
+    auto lds_load = [&](float4(&w)[8], float4(&x)[8], int k) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        w[q] = *reinterpret_cast<const float4*>(wrow + k + 4 * q);
+        x[q] = *reinterpret_cast<const float4*>(xrow + k + 4 * q);
+      }
+    };
+    auto chain = [&](const float4(&w)[8], const float4(&x)[8]) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        if constexpr (EPV == 8) {
+          acc = __builtin_fmaf(x[q].x, w[q].x, acc);
+          acc = __builtin_fmaf(x[q].y, w[q].y, acc);
+          acc = __builtin_fmaf(x[q].z, w[q].z, acc);
+          acc = __builtin_fmaf(x[q].w, w[q].w, acc);
+        } else {
+          acc = __fadd_rn(acc, __fmul_rn(x[q].x, w[q].x));
+          acc = __fadd_rn(acc, __fmul_rn(x[q].y, w[q].y));
+          acc = __fadd_rn(acc, __fmul_rn(x[q].z, w[q].z));
+          acc = __fadd_rn(acc, __fmul_rn(x[q].w, w[q].w));
+        }
+      }
+    };
+    lds_load(wa, xa, 0);
+    for (int k = 0; k < n; k += 64) {
+      lds_load(wb, xb, k + 32);
+      __builtin_amdgcn_sched_barrier(0);
+      chain(wa, xa);
+      __builtin_amdgcn_sched_barrier(0);
+      if (k + 64 < n) lds_load(wa, xa, k + 64);
+      __builtin_amdgcn_sched_barrier(0);
+      chain(wb, xb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+#pragma unroll
+  for (int j = 0; j < PF; ++j) issue(wr[j], xr[j], j * ROUTER_KC);
+  for (int c0 = 0; c0 < H; c0 += PF * ROUTER_KC) {
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+      const int cj = c0 + j * ROUTER_KC;
+      if (cj < H) {
+        const int n = min(ROUTER_KC, H - cj);
+        stage(wr[j], xr[j], n);
+        lds_wave_sync();
+        issue(wr[j], xr[j], cj + PF * ROUTER_KC);
+        consume(n);
+        lds_wave_sync();
       }
     }
   }
 
-  // Candidate keys: (order-preserving value bits, inverted index) so that the
-  // wave maximum is the largest value and, among equals, the lowest index.
-  // Values that the reference's strict '>' against lowest() never admits
-  // (NaN, -inf, -FLT_MAX) get key 0.
+  const bool valid = (t < T) && (e < E);
+  if (valid) {
+    float v = acc;
+    if (p.bias != nullptr) v = __fadd_rn(v, as_global(p.bias)[e]);
+    stc(&p.cand[static_cast<size_t>(t) * E + e], make_key(v, e, true));
+  }
+  fence_release();
+  if (ei == 0 && t < T) add_relaxed(&p.tok_arrive[t], 1u);
+}
+
+// All expert groups of token t have left their keys: pick the winners.
+__device__ __noinline__ void router_select_task(const Params& p, int t) {
+  constexpr int MAXEPL = MAX_EXPERTS / 64;
+  const int lane = lane_id();
   unsigned long long key[MAXEPL];
 #pragma unroll
   for (int j = 0; j < MAXEPL; ++j) {
     const int e = lane + 64 * j;
-    float v = acc[j];
-    if (p.bias != nullptr && e < p.E) v = __fadd_rn(v, p.bias[e]);
-    const bool valid = (j < epl) && (e < p.E) && (v > -FLT_MAX);
-    unsigned u = __float_as_uint(v);
-    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-    key[j] = valid ? ((static_cast<unsigned long long>(u) << 32) |
-                      static_cast<unsigned long long>(0xFFFFFFFFu - static_cast<unsigned>(e)))
-                   : 0ull;
+    key[j] = e < p.E ? ldc(&p.cand[static_cast<size_t>(t) * p.E + e]) : 0ull;
   }
-
-  int my_idx = -1;
-  float my_val = -FLT_MAX;
-  for (int s = 0; s < p.K; ++s) {
-    unsigned long long best = key[0];
-#pragma unroll
-    for (int j = 1; j < MAXEPL; ++j) best = key[j] > best ? key[j] : best;
-    best = wave_max_u64(best);
-    int e = -1;
-    float v = -FLT_MAX;
-    if (best != 0ull) {
-      e = static_cast<int>(0xFFFFFFFFu - static_cast<unsigned>(best & 0xFFFFFFFFull));
-      unsigned u = static_cast<unsigned>(best >> 32);
-      u = (u & 0x80000000u) ? (u & 0x7FFFFFFFu) : ~u;
-      v = __uint_as_float(u);
-#pragma unroll
-      for (int j = 0; j < MAXEPL; ++j)
-        if (e == lane + 64 * j) key[j] = 0ull;
-    }
-    if (lane == s) {
-      my_idx = e;
-      my_val = v;
-    }
-  }
-
-  // softmax over the K winners (descending, so the first is the maximum)
-  const double v0 = static_cast<double>(__shfl(my_val, 0, 64));
-  const double ex = lane < p.K ? exp(static_cast<double>(my_val) - v0) : 0.0;
-  double sum = 0.0;
-  for (int s = 0; s < p.K; ++s) sum += __shfl(ex, s, 64);
-  if (lane < p.K) {
-    float w;
-    if (sum <= 0.0) {
-      w = static_cast<float>(1.0 / static_cast<double>(p.K));
-    } else {
-      w = static_cast<float>(ex / sum);
-    }
-    p.topk_idx[static_cast<size_t>(t) * p.K + lane] = my_idx;
-    p.topk_w[static_cast<size_t>(t) * p.K + lane] = w;
-    if (my_idx >= 0) {
-      __hip_atomic_fetch_or(&p.masks[static_cast<size_t>(my_idx) * p.W + (t >> 6)],
-                            1ull << (t & 63), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-  wave_signal(&p.ctl->router_done);
+  if (lane == 0) stc(&p.tok_arrive[t], 0u);
+  router_select(p, t, key);
+  wave_arrive(&p.ctl->router_done.v);
 }
 
-// ----------------------------------------------------------------------- scan
+// ------------------------------------------------------------- scan / scatter
+// The tables the scan and scatter tasks work on, held in registers (Params is
+// reached through a generic reference, which every store would force the
+// compiler to re-read).
+struct RouteTables {
+  int T, E, K, W, max_mtiles;
+  int* topk_idx;
+  float* topk_w;
+  unsigned long long* masks;
+  int* word_prefix;
+  int* expert_count;
+  int* expert_offset;
+  int* perm;
+  float* row_w;
+  TileDesc* mtiles;
+};
+__device__ __forceinline__ RouteTables route_tables(const Params& p) {
+  RouteTables r;
+  r.T = p.T;
+  r.E = p.E;
+  r.K = p.K;
+  r.W = p.W;
+  r.max_mtiles = p.max_mtiles;
+  r.topk_idx = p.topk_idx;
+  r.topk_w = p.topk_w;
+  r.masks = p.masks;
+  r.word_prefix = p.word_prefix;
+  r.expert_count = p.expert_count;
+  r.expert_offset = p.expert_offset;
+  r.perm = p.perm;
+  r.row_w = p.row_w;
+  r.mtiles = p.mtiles;
+  return r;
+}
+
+// Permuted row of assignment i = t*K+slot: rows of one expert ascend by token.
+__device__ __forceinline__ void scatter_entry(const RouteTables& r, int i) {
+  const int e = ldc(&r.topk_idx[i]);
+  if (e >= 0) {
+    const int t = i / r.K;
+    const int wd = t >> 6;
+    const unsigned long long m = ldc(&r.masks[static_cast<size_t>(e) * r.W + wd]);
+    const unsigned long long below = m & ((1ull << (t & 63)) - 1ull);
+    const int pos = ldc(&r.expert_offset[e]) +
+                    ldc(&r.word_prefix[static_cast<size_t>(e) * r.W + wd]) + __popcll(below);
+    stc(&r.perm[pos], i);
+    stc(&r.row_w[pos], ldc(&r.topk_w[i]));
+  }
+}
+
 // Expert counts and offsets from the selection bit masks, and the table of row
 // tiles. The permutation this defines is the stable sort of (token, slot) by
 // expert id: inside an expert, rows ascend by token id. The reference has no
 // permutation stage (it runs one GEMV per (token, slot)); this is the
-// token-grouping the streaming and tiled GEMMs need.
-__device__ void scan_task(const Params& p) {
-  constexpr int MAXEPL = MAX_EXPERTS / 64;
+// token-grouping the streaming and tiled GEMMs need. For small batches the same
+// wave also writes the permutation.
+__device__ __noinline__ void scan_task(const Params& p) {
+  const RouteTables r = route_tables(p);
+  const int fuse = p.fuse_scatter;
+  Control* ctl = p.ctl;
   const int lane = lane_id();
-  const int epl = (p.E + 63) >> 6;
-  const int wact = (p.T + 63) >> 6;
+  const int epl = (r.E + 63) >> 6;
+  const int wact = (r.T + 63) >> 6;
   int base = 0, tile_base = 0;
   for (int j = 0; j < epl; ++j) {
     const int e = lane + 64 * j;
     int c = 0;
-    if (e < p.E) {
-      const unsigned long long* m = p.masks + static_cast<size_t>(e) * p.W;
-      int* wp = p.word_prefix + static_cast<size_t>(e) * p.W;
+    if (e < r.E) {
+      const unsigned long long* m = r.masks + static_cast<size_t>(e) * r.W;
+      int* wp = r.word_prefix + static_cast<size_t>(e) * r.W;
       for (int w = 0; w < wact; ++w) {
-        wp[w] = c;
-        c += __popcll(m[w]);
+        stc(&wp[w], c);
+        c += __popcll(ldc(&m[w]));
       }
     }
     const int incl = wave_inclusive_scan(c);
@@ -301,17 +592,14 @@ __device__ void scan_task(const Params& p) {
     const int nt = (c + SKINNY_MT - 1) / SKINNY_MT;
     const int tincl = wave_inclusive_scan(nt);
     const int toff = tile_base + tincl - nt;
-    if (e < p.E) {
-      p.expert_count[e] = c;
-      p.expert_offset[e] = off;
+    if (e < r.E) {
+      stc(&r.expert_count[e], c);
+      stc(&r.expert_offset[e], off);
       for (int i = 0; i < nt; ++i) {
-        if (toff + i < p.max_mtiles) {
-          TileDesc d;
-          d.expert = e;
-          d.row0 = off + i * SKINNY_MT;
-          d.rows = min(SKINNY_MT, c - i * SKINNY_MT);
-          d.pad = 0;
-          p.mtiles[toff + i] = d;
+        if (toff + i < r.max_mtiles) {
+          stc16(&r.mtiles[toff + i],
+                make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + i * SKINNY_MT),
+                           static_cast<unsigned>(min(SKINNY_MT, c - i * SKINNY_MT)), 0u));
         }
       }
     }
@@ -319,57 +607,94 @@ __device__ void scan_task(const Params& p) {
     tile_base += __shfl(tincl, 63, 64);
   }
   if (lane == 0) {
-    p.expert_offset[p.E] = base;
-    if (tile_base > p.max_mtiles) {
-      __hip_atomic_fetch_or(&p.ctl->error, ERR_CAPACITY, __ATOMIC_RELAXED,
-                            __HIP_MEMORY_SCOPE_AGENT);
+    stc(&r.expert_offset[r.E], base);
+    if (tile_base > r.max_mtiles) {
+      or_relaxed(&ctl->error.v, ERR_CAPACITY);
       tile_base = 0;
     }
-    p.ctl->n_mtiles = static_cast<unsigned>(tile_base);
+    stc(&ctl->n_mtiles.v, static_cast<unsigned>(tile_base));
   }
-  wave_signal(&p.ctl->scan_done);
+  fence_release();
+  broadcast_flag(p, FLAG_SCAN);
+  if (fuse) {
+    // offsets and prefixes were written by other lanes of this wave; the
+    // release above has waited for those stores
+    const int n = r.T * r.K;
+    constexpr int B = 8;  // entries per lane whose loads are in flight together
+    for (int i0 = lane; i0 < n; i0 += 64 * B) {
+      int ee[B], off[B], pre[B];
+      unsigned long long mm[B];
+      float ww[B];
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int i = i0 + 64 * b;
+        ee[b] = i < n ? ldc(&r.topk_idx[i]) : -1;
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        if (ee[b] >= 0) {
+          const int i = i0 + 64 * b;
+          const int wd = (i / r.K) >> 6;
+          mm[b] = ldc(&r.masks[static_cast<size_t>(ee[b]) * r.W + wd]);
+          off[b] = ldc(&r.expert_offset[ee[b]]);
+          pre[b] = ldc(&r.word_prefix[static_cast<size_t>(ee[b]) * r.W + wd]);
+          ww[b] = ldc(&r.topk_w[i]);
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        if (ee[b] >= 0) {
+          const int i = i0 + 64 * b;
+          const int t = i / r.K;
+          const int pos = off[b] + pre[b] + __popcll(mm[b] & ((1ull << (t & 63)) - 1ull));
+          stc(&r.perm[pos], i);
+          stc(&r.row_w[pos], ww[b]);
+        }
+      }
+    }
+    fence_release();
+    broadcast_flag(p, FLAG_PERM);
+  }
 }
 
-// -------------------------------------------------------------------- scatter
 __device__ void scatter_task(const Params& p, int t) {
+  const RouteTables r = route_tables(p);
   const int lane = lane_id();
-  if (lane < p.K) {
-    const int e = p.topk_idx[static_cast<size_t>(t) * p.K + lane];
-    if (e >= 0) {
-      const int wd = t >> 6;
-      const unsigned long long m = p.masks[static_cast<size_t>(e) * p.W + wd];
-      const unsigned long long below = m & ((1ull << (t & 63)) - 1ull);
-      const int pos = p.expert_offset[e] + p.word_prefix[static_cast<size_t>(e) * p.W + wd] +
-                      __popcll(below);
-      p.perm[pos] = t * p.K + lane;
-      p.row_w[pos] = p.topk_w[static_cast<size_t>(t) * p.K + lane];
-    }
-  }
-  wave_signal(&p.ctl->perm_done);
+  if (lane < r.K) scatter_entry(r, t * r.K + lane);
+  const unsigned old = wave_arrive(&p.ctl->perm_done.v);
+  if (old == static_cast<unsigned>(r.T) - 1u) broadcast_flag(p, FLAG_PERM);
 }
 
 // ------------------------------------------------- streaming 16x16 MFMA sweep
 // acc[i][r] += A_i (16 weight rows) . B_r (16 token rows)^T over `ksteps` steps
 // of 4*EPV elements. ap[i] / bp[r] already point at this lane's row and
-// k-offset. Fragments are double-buffered in registers, U steps per buffer, so
-// the next buffer's loads are in flight while the current one feeds the MFMAs.
-template <typename DT, int NA, int RB, int U>
-__device__ __forceinline__ void stream_mma(const typename DT::elem* const (&ap)[NA],
+// k-offset. Each round issues U steps' worth of 16-byte loads and then feeds
+// the MFMAs; the other waves of the CU keep HBM busy meanwhile. `pre` runs once
+// after the first round's weight loads are in flight and before any B row is
+// touched (the down projection waits for its h rows there).
+template <typename DT, int NA, int RB, int U, bool COH_B, typename Pre>
+__device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[NA],
                                            const typename DT::elem* const (&bp)[RB], int ksteps,
-                                           f32x4 (&acc)[NA][RB]) {
+                                           f32x4 (&acc)[NA][RB], Pre pre) {
   constexpr int KS = 4 * DT::EPV;
-  uint4 a0[U][NA], b0[U][RB], a1[U][NA], b1[U][RB];
+  uint4 a[U][NA], b[U][RB];
 
-  auto load = [&](uint4(&a)[U][NA], uint4(&b)[U][RB], int s) {
+  auto load_a = [&](int s) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
+    for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int i = 0; i < NA; ++i) a[u][i] = ld16(ap[i] + static_cast<size_t>(s + u) * KS);
-#pragma unroll
-      for (int r = 0; r < RB; ++r) b[u][r] = ld16(bp[r] + static_cast<size_t>(s + u) * KS);
-    }
   };
-  auto mma = [&](uint4(&a)[U][NA], uint4(&b)[U][RB]) {
+  auto load_b = [&](int s) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < RB; ++r) {
+        const typename DT::elem* q = bp[r] + static_cast<size_t>(s + u) * KS;
+        b[u][r] = COH_B ? ldc16(q) : ld16(q);
+      }
+  };
+  auto mma = [&]() {
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -381,27 +706,35 @@ __device__ __forceinline__ void stream_mma(const typename DT::elem* const (&ap)[
   const int main_steps = (ksteps / U) * U;
   int s = 0;
   if (main_steps > 0) {
-    load(a0, b0, 0);
-    for (; s + 2 * U <= main_steps; s += 2 * U) {
-      load(a1, b1, s + U);
-      mma(a0, b0);
-      if (s + 2 * U < main_steps) load(a0, b0, s + 2 * U);
-      mma(a1, b1);
-    }
-    if (s < main_steps) {
-      mma(a0, b0);
-      s += U;
-    }
+    load_a(0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (!pre()) return false;
+    load_b(0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma();
+    s = U;
+  } else {
+    if (!pre()) return false;
+  }
+  for (; s < main_steps; s += U) {
+    __builtin_amdgcn_sched_barrier(0);
+    load_a(s);
+    load_b(s);
+    __builtin_amdgcn_sched_barrier(0);
+    mma();
   }
   for (; s < ksteps; ++s) {  // remainder when ksteps is not a multiple of U
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      const uint4 a = ld16(ap[i] + static_cast<size_t>(s) * KS);
+      const uint4 av = ld16(ap[i] + static_cast<size_t>(s) * KS);
 #pragma unroll
-      for (int r = 0; r < RB; ++r)
-        acc[i][r] = mma16<DT>(a, ld16(bp[r] + static_cast<size_t>(s) * KS), acc[i][r]);
+      for (int r = 0; r < RB; ++r) {
+        const typename DT::elem* q = bp[r] + static_cast<size_t>(s) * KS;
+        acc[i][r] = mma16<DT>(av, COH_B ? ldc16(q) : ld16(q), acc[i][r]);
+      }
     }
   }
+  return true;
 }
 
 __device__ __forceinline__ float silu_mul(float a, float b) {
@@ -417,16 +750,23 @@ __device__ __forceinline__ float silu_mul(float a, float b) {
   return a * s * b;
 }
 
+// Steps per load round, by rows blocks of the tile: keeps a round near 32-40
+// loads of 16 bytes per lane.
+template <int NA, int RB>
+struct RoundSteps {
+  static constexpr int value = RB == 1 ? (NA <= 2 ? 16 : 8) : (RB == 2 ? (NA <= 2 ? 8 : 4) : (NA <= 2 ? 4 : 2));
+};
+
 // -------------------------------------------------------------------- gate/up
-// h[row, n0 .. n0+32) for the rows of one tile. Follows
+// h[row, n0 .. n0+16*G1_NB) for the rows of one tile. Follows
 // refExpertFFN1.h:51-65 (two GEMMs against the [2I,H] expert matrix, then
 // SiLU(gate) * up), accumulated on MFMA in float.
 template <typename DT, int RB>
-__device__ void gateup_task(const Params& p, const TileDesc& tile, int nblk) {
+__device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile, int nblk) {
   typedef typename DT::elem elem;
   constexpr int EPV = DT::EPV;
   constexpr int NA = 2 * G1_NB;
-  constexpr int U = RB >= 4 ? 1 : (RB == 2 ? 2 : 3);
+  constexpr int U = RoundSteps<NA, RB>::value;
   const int lane = lane_id();
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = nblk * (16 * G1_NB);
@@ -436,14 +776,14 @@ __device__ void gateup_task(const Params& p, const TileDesc& tile, int nblk) {
   const elem* ap[NA];
 #pragma unroll
   for (int b = 0; b < G1_NB; ++b) {
-    ap[b] = w13 + static_cast<size_t>(n0 + 16 * b + r16) * p.H + g * EPV;            // gate rows
-    ap[G1_NB + b] = w13 + static_cast<size_t>(p.I + n0 + 16 * b + r16) * p.H + g * EPV;  // up rows
+    ap[b] = w13 + static_cast<size_t>(n0 + 16 * b + r16) * p.H + g * EPV;                // gate
+    ap[G1_NB + b] = w13 + static_cast<size_t>(p.I + n0 + 16 * b + r16) * p.H + g * EPV;  // up
   }
   const elem* bp[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
     const int row = min(r * 16 + r16, tile.rows - 1);
-    const int tok = p.perm[tile.row0 + row] / p.K;
+    const int tok = ldc(&p.perm[tile.row0 + row]) / p.K;
     bp[r] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(tok) * p.H + g * EPV;
   }
   f32x4 acc[NA][RB];
@@ -452,7 +792,7 @@ __device__ void gateup_task(const Params& p, const TileDesc& tile, int nblk) {
 #pragma unroll
     for (int r = 0; r < RB; ++r) acc[i][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  stream_mma<DT, NA, RB, U>(ap, bp, p.H / (4 * EPV), acc);
+  stream_mma<DT, NA, RB, U, false>(ap, bp, p.H / (4 * EPV), acc, [] { return true; });
 
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
@@ -465,13 +805,14 @@ __device__ void gateup_task(const Params& p, const TileDesc& tile, int nblk) {
         for (int v = 0; v < 4; ++v) hv[v] = silu_mul(acc[b][r][v], acc[G1_NB + b][r][v]);
         const size_t off = static_cast<size_t>(tile.row0 + row) * p.I + n0 + 16 * b + 4 * g;
         if constexpr (EPV == 8) {
-          uint2 pk;
-          pk.x = f2bf(hv[0]) | (f2bf(hv[1]) << 16);
-          pk.y = f2bf(hv[2]) | (f2bf(hv[3]) << 16);
-          *reinterpret_cast<uint2*>(reinterpret_cast<unsigned short*>(p.h) + off) = pk;
+          const unsigned lo = f2bf(hv[0]) | (f2bf(hv[1]) << 16);
+          const unsigned hi = f2bf(hv[2]) | (f2bf(hv[3]) << 16);
+          stc(reinterpret_cast<unsigned long long*>(reinterpret_cast<unsigned short*>(p.h) + off),
+              static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32));
         } else {
-          *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.h) + off) =
-              make_float4(hv[0], hv[1], hv[2], hv[3]);
+          stc16(reinterpret_cast<float*>(p.h) + off,
+                make_uint4(__float_as_uint(hv[0]), __float_as_uint(hv[1]), __float_as_uint(hv[2]),
+                           __float_as_uint(hv[3])));
         }
       }
     }
@@ -479,15 +820,18 @@ __device__ void gateup_task(const Params& p, const TileDesc& tile, int nblk) {
 }
 
 // ----------------------------------------------------------------------- down
-// y[t*K+slot, n0 .. n0+64) = w * (h[row] . W2[e]^T): refFullMoe.h:58-65 with the
-// gate weight applied before the slot sum, as the reference GPU path does
-// (src/hip/kernel/tasks/ffn2Task.h:37-40).
+// y[t*K+slot, n0 .. n0+16*G2_NB) = w * (h[row] . W2[e]^T): refFullMoe.h:58-65
+// with the gate weight applied before the slot sum, as the reference GPU path
+// does (src/hip/kernel/tasks/ffn2Task.h:37-40). The weight rows do not depend
+// on h, so their first loads are issued before the wait for the tile's
+// gate/up tasks. Returns false if that wait failed.
 template <typename DT, int RB>
-__device__ void down_task(const Params& p, const TileDesc& tile, int nblk) {
+__device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, int nblk, unsigned* dep,
+                          unsigned dep_target) {
   typedef typename DT::elem elem;
   constexpr int EPV = DT::EPV;
   constexpr int NA = G2_NB;
-  constexpr int U = RB >= 4 ? 1 : (RB == 2 ? 2 : 3);
+  constexpr int U = RoundSteps<NA, RB>::value;
   const int lane = lane_id();
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = nblk * (16 * G2_NB);
@@ -509,21 +853,26 @@ __device__ void down_task(const Params& p, const TileDesc& tile, int nblk) {
 #pragma unroll
     for (int r = 0; r < RB; ++r) acc[i][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  stream_mma<DT, NA, RB, U>(ap, bp, p.I / (4 * EPV), acc);
+  const bool ok = stream_mma<DT, NA, RB, U, true>(ap, bp, p.I / (4 * EPV), acc, [&] {
+    return wave_wait_ge(dep, dep_target, p.ctl, p.spin_limit);
+  });
+  if (!ok) return false;
 
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
     const int row = r * 16 + r16;
     if (row < tile.rows) {
-      const float w = p.row_w[tile.row0 + row];
-      const size_t dst = static_cast<size_t>(p.perm[tile.row0 + row]) * p.H;
+      const float w = ldc(&p.row_w[tile.row0 + row]);
+      const size_t dst = static_cast<size_t>(ldc(&p.perm[tile.row0 + row])) * p.H;
 #pragma unroll
       for (int b = 0; b < NA; ++b) {
-        *reinterpret_cast<float4*>(p.y + dst + n0 + 16 * b + 4 * g) =
-            make_float4(acc[b][r][0] * w, acc[b][r][1] * w, acc[b][r][2] * w, acc[b][r][3] * w);
+        stc16(p.y + dst + n0 + 16 * b + 4 * g,
+              make_uint4(__float_as_uint(acc[b][r][0] * w), __float_as_uint(acc[b][r][1] * w),
+                         __float_as_uint(acc[b][r][2] * w), __float_as_uint(acc[b][r][3] * w)));
       }
     }
   }
+  return true;
 }
 
 // -------------------------------------------------------------------- combine
@@ -536,13 +885,12 @@ __device__ void combine_task(const Params& p, int t, int chunk) {
   if (c < p.H) {
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int k = 0; k < p.K; ++k) {
-      if (p.topk_idx[static_cast<size_t>(t) * p.K + k] < 0) continue;
-      const float4 v =
-          *reinterpret_cast<const float4*>(p.y + (static_cast<size_t>(t) * p.K + k) * p.H + c);
-      s.x += v.x;
-      s.y += v.y;
-      s.z += v.z;
-      s.w += v.w;
+      if (ldc(&p.topk_idx[static_cast<size_t>(t) * p.K + k]) < 0) continue;
+      const uint4 v = ldc16(p.y + (static_cast<size_t>(t) * p.K + k) * p.H + c);
+      s.x += __uint_as_float(v.x);
+      s.y += __uint_as_float(v.y);
+      s.z += __uint_as_float(v.z);
+      s.w += __uint_as_float(v.w);
     }
     const size_t off = static_cast<size_t>(t) * p.H + c;
     if constexpr (DT::EPV == 8) {
@@ -554,43 +902,130 @@ __device__ void combine_task(const Params& p, int t, int chunk) {
       *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.out) + off) = s;
     }
   }
-  // the selection masks are dead once every scatter task has run: clear this
+  // the selection masks are dead once the permutation is written: clear this
   // token block's words for the next launch
   if (chunk == 0 && (t & 63) == 0) {
-    for (int e = lane; e < p.E; e += 64) p.masks[static_cast<size_t>(e) * p.W + (t >> 6)] = 0ull;
+    for (int e = lane; e < p.E; e += 64) stc(&p.masks[static_cast<size_t>(e) * p.W + (t >> 6)], 0ull);
   }
+}
+
+// Wave-uniform bounded wait for this workgroup's copy of a phase flag. Only one
+// wave of the workgroup polls HBM; the others watch a word in LDS that the
+// polling wave sets (1 = flag seen, 2 = failed).
+__device__ __forceinline__ bool wait_flag(const Params& p, int which, unsigned* lds_flag,
+                                          unsigned* lds_poller) {
+  int ok = 1;
+  if (lane_id() == 0) {
+    while (true) {
+      const unsigned f = __hip_atomic_load(&lds_flag[which], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (f != 0u) {
+        ok = f == 1u;
+        break;
+      }
+      if (__hip_atomic_exchange(&lds_poller[which], 1u, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_WORKGROUP) == 0u) {
+        // this wave polls for the workgroup
+        const unsigned* g = &p.wgflags[blockIdx.x].f[which];
+        const long long t0 = wall_clock64();
+        unsigned spins = 0;
+        unsigned res = 1u;
+        while (ld_relaxed(g) == 0u) {
+          if ((++spins & 31u) == 0u && ld_relaxed(&p.ctl->error.v) != 0u) {
+            res = 2u;
+            break;
+          }
+          if (wall_clock64() - t0 > p.spin_limit) {
+            or_relaxed(&p.ctl->error.v, ERR_TIMEOUT);
+            res = 2u;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(16);
+        }
+        __hip_atomic_store(&lds_flag[which], res, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        ok = res == 1u;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+  }
+  ok = __builtin_amdgcn_readfirstlane(ok);
+  fence_acquire();
+  return ok != 0;
 }
 
 // ---------------------------------------------------------------- worker loop
 template <typename DT>
 __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
+  __shared__ unsigned lds_flag[4];
+  __shared__ unsigned lds_poller[4];
+  if (threadIdx.x < 4) {
+    lds_flag[threadIdx.x] = 0u;
+    lds_poller[threadIdx.x] = 0u;
+  }
+  __syncthreads();
   const int lane = lane_id();
+  const int wave_in_group = threadIdx.x >> 6;
+  const int waves_per_group = blockDim.x >> 6;
   Control* ctl = p.ctl;
   const unsigned T = static_cast<unsigned>(p.T);
-  const unsigned t_scan = T, t_scatter0 = T + 1u, t_dyn0 = 2u * T + 1u;
+  const unsigned n_eg = static_cast<unsigned>((p.E + ROUTER_EXP - 1) / ROUTER_EXP);
+  const unsigned n_tg = (T + ROUTER_TOK - 1u) / ROUTER_TOK;
+  const unsigned n_dot = n_tg * n_eg;
+  const unsigned n_router = n_dot + T;  // dot tasks, then one select task per token
+  const unsigned t_scan = n_router;
+  const unsigned t_scatter0 = n_router + 1u;
+  const unsigned t_dyn0 = t_scatter0 + (p.fuse_scatter ? 0u : T);
   const unsigned nt1 = static_cast<unsigned>(p.I / (16 * G1_NB));
   const unsigned nt2 = static_cast<unsigned>(p.H / (16 * G2_NB));
   const unsigned ncomb = static_cast<unsigned>((p.H + COMBINE_COLS - 1) / COMBINE_COLS);
+  const unsigned worker = blockIdx.x * waves_per_group + wave_in_group;
   unsigned n1 = 0, n2 = 0, nc = 0;
   bool have_dyn = false, perm_ready = false, g2_ready = false;
 
-  while (true) {
-    unsigned tk = 0;
-    if (lane == 0) tk = add_relaxed(&ctl->ticket, 1u);
-    tk = __builtin_amdgcn_readfirstlane(tk);
+  // The first ticket of every worker is fixed (wave w of every workgroup before
+  // wave w+1 of any, so the first tasks spread over all CUs); the shared counter
+  // hands out the tickets after those.
+  const unsigned n_workers = static_cast<unsigned>(p.n_workers);
+  bool first = true;
 
-    if (tk < T) {
-      router_task<DT>(p, static_cast<int>(tk));
+  while (true) {
+    const long long t_fetch = p.trace ? wall_clock64() : 0;
+    unsigned tk = static_cast<unsigned>(wave_in_group) * gridDim.x + blockIdx.x;
+    if (!first) {
+      if (lane == 0) tk = n_workers + add_relaxed(&ctl->ticket.v, 1u);
+      tk = __builtin_amdgcn_readfirstlane(tk);
+    }
+    first = false;
+    unsigned kind = 0, aux = 0;
+    long long t_ready = 0;
+
+    if (tk < n_dot) {
+      kind = 0;
+      aux = tk;
+      if (p.trace) t_ready = wall_clock64();
+      router_dot_task<DT>(p, static_cast<int>(tk / n_eg), static_cast<int>(tk % n_eg));
+    } else if (tk < n_router) {
+      kind = 6;
+      aux = tk - n_dot;
+      if (!wave_wait_ge(&p.tok_arrive[aux], n_eg, ctl, p.spin_limit)) break;
+      if (p.trace) t_ready = wall_clock64();
+      router_select_task(p, static_cast<int>(aux));
     } else if (tk == t_scan) {
-      if (!wave_wait_ge(&ctl->router_done, T, ctl, p.spin_limit)) break;
+      kind = 1;
+      if (!wave_wait_ge(&ctl->router_done.v, T, ctl, p.spin_limit)) break;
+      if (p.trace) t_ready = wall_clock64();
       scan_task(p);
     } else if (tk < t_dyn0) {
-      if (!wave_wait_ge(&ctl->scan_done, 1u, ctl, p.spin_limit)) break;
-      scatter_task(p, static_cast<int>(tk - t_scatter0));
+      kind = 2;
+      aux = tk - t_scatter0;
+      if (!wait_flag(p, FLAG_SCAN, lds_flag, lds_poller)) break;
+      if (p.trace) t_ready = wall_clock64();
+      scatter_task(p, static_cast<int>(aux));
     } else {
       if (!have_dyn) {
-        if (!wave_wait_ge(&ctl->scan_done, 1u, ctl, p.spin_limit)) break;
-        const unsigned nm = ctl->n_mtiles;
+        if (!wait_flag(p, FLAG_SCAN, lds_flag, lds_poller)) break;
+        const unsigned nm = ldc(&ctl->n_mtiles.v);
         n1 = nm * nt1;
         n2 = nm * nt2;
         nc = T * ncomb;
@@ -598,11 +1033,14 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
       }
       const unsigned j = tk - t_dyn0;
       if (j < n1) {
+        kind = 3;
+        aux = j / nt1;
         if (!perm_ready) {
-          if (!wave_wait_ge(&ctl->perm_done, T, ctl, p.spin_limit)) break;
+          if (!wait_flag(p, FLAG_PERM, lds_flag, lds_poller)) break;
           perm_ready = true;
         }
-        const TileDesc tile = p.mtiles[j / nt1];
+        if (p.trace) t_ready = wall_clock64();
+        const TileDesc tile = ld_tile(&p.mtiles[aux]);
         const int nblk = static_cast<int>(j % nt1);
         if (tile.rows <= 16) {
           gateup_task<DT, 1>(p, tile, nblk);
@@ -611,55 +1049,75 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
         } else {
           gateup_task<DT, 4>(p, tile, nblk);
         }
-        wave_signal(&p.g1_done[j / nt1]);
+        wave_arrive(&p.g1_done[aux].v);
       } else if (j < n1 + n2) {
-        const unsigned m = (j - n1) / nt2;
+        kind = 4;
+        aux = (j - n1) / nt2;
         const int nblk = static_cast<int>((j - n1) % nt2);
-        if (!wave_wait_ge(&p.g1_done[m], nt1, ctl, p.spin_limit)) break;
-        const TileDesc tile = p.mtiles[m];
+        if (p.trace) t_ready = wall_clock64();
+        const TileDesc tile = ld_tile(&p.mtiles[aux]);
+        unsigned* dep = &p.g1_done[aux].v;
+        bool ok;
         if (tile.rows <= 16) {
-          down_task<DT, 1>(p, tile, nblk);
+          ok = down_task<DT, 1>(p, tile, nblk, dep, nt1);
         } else if (tile.rows <= 32) {
-          down_task<DT, 2>(p, tile, nblk);
+          ok = down_task<DT, 2>(p, tile, nblk, dep, nt1);
         } else {
-          down_task<DT, 4>(p, tile, nblk);
+          ok = down_task<DT, 4>(p, tile, nblk, dep, nt1);
         }
-        wave_signal(&ctl->g2_done);
+        if (!ok) break;
+        const unsigned old = wave_arrive(&ctl->g2_done.v);
+        if (old == n2 - 1u) broadcast_flag(p, FLAG_G2);
       } else if (j < n1 + n2 + nc) {
+        kind = 5;
         if (!g2_ready) {
-          if (!wave_wait_ge(&ctl->g2_done, n2, ctl, p.spin_limit)) break;
+          if (n2 != 0u && !wait_flag(p, FLAG_G2, lds_flag, lds_poller)) break;
           g2_ready = true;
         }
+        if (p.trace) t_ready = wall_clock64();
         const unsigned q = j - n1 - n2;
+        aux = q / ncomb;
         combine_task<DT>(p, static_cast<int>(q / ncomb), static_cast<int>(q % ncomb));
       } else {
         break;
       }
+    }
+    if (p.trace && lane == 0 && tk < p.trace_cap) {
+      const long long t_end = wall_clock64();
+      TraceRec* r = p.trace + tk;  // 48 bytes: four words, then four 64-bit times
+      st16(r, u32x4{tk, kind, worker, aux});
+      st16(reinterpret_cast<char*>(r) + 16,
+           u32x4{static_cast<unsigned>(t_fetch), static_cast<unsigned>(t_fetch >> 32),
+                 static_cast<unsigned>(t_ready), static_cast<unsigned>(t_ready >> 32)});
+      st16(reinterpret_cast<char*>(r) + 32,
+           u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), 0u, 0u});
     }
   }
 
   // The last worker out returns every counter to zero for the next launch.
   unsigned last = 0;
   if (lane == 0) {
-    last = (__hip_atomic_fetch_add(&ctl->exit_count, 1u, __ATOMIC_ACQ_REL,
-                                   __HIP_MEMORY_SCOPE_AGENT) ==
-            static_cast<unsigned>(p.n_workers) - 1u)
+    last = (add_relaxed(&ctl->exit_count.v, 1u) == static_cast<unsigned>(p.n_workers) - 1u)
                ? 1u
                : 0u;
   }
   last = __builtin_amdgcn_readfirstlane(last);
   if (last) {
-    const unsigned nm = min(ctl->n_mtiles, static_cast<unsigned>(p.max_mtiles));
-    for (unsigned i = lane; i < nm; i += 64) p.g1_done[i] = 0u;
+    const unsigned nm = min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
+    for (unsigned i = lane; i < nm; i += 64) stc(&p.g1_done[i].v, 0u);
+    for (int g = lane; g < p.n_groups; g += 64) {
+      stc(&p.wgflags[g].f[FLAG_SCAN], 0u);
+      stc(&p.wgflags[g].f[FLAG_PERM], 0u);
+      stc(&p.wgflags[g].f[FLAG_G2], 0u);
+    }
     if (lane == 0) {
-      ctl->launches = ctl->launches + 1u;
-      ctl->router_done = 0u;
-      ctl->scan_done = 0u;
-      ctl->perm_done = 0u;
-      ctl->g2_done = 0u;
-      ctl->n_mtiles = 0u;
-      ctl->exit_count = 0u;
-      ctl->ticket = 0u;
+      stc(&ctl->launches.v, ldc(&ctl->launches.v) + 1u);
+      stc(&ctl->router_done.v, 0u);
+      stc(&ctl->perm_done.v, 0u);
+      stc(&ctl->g2_done.v, 0u);
+      stc(&ctl->n_mtiles.v, 0u);
+      stc(&ctl->exit_count.v, 0u);
+      stc(&ctl->ticket.v, 0u);
     }
   }
 }
@@ -668,12 +1126,24 @@ template __global__ void moe_stream_kernel<F32>(const Params);
 template __global__ void moe_stream_kernel<BF16>(const Params);
 
 hipError_t launch_stream_kernel(const Params& p, int dtype, int grid, hipStream_t stream) {
+  const size_t lds = static_cast<size_t>(8) * ROUTER_LDS_FLOATS * sizeof(float);
   if (dtype == DT_BF16) {
-    hipLaunchKernelGGL(moe_stream_kernel<BF16>, dim3(grid), dim3(512), 0, stream, p);
+    hipLaunchKernelGGL(moe_stream_kernel<BF16>, dim3(grid), dim3(512), lds, stream, p);
   } else {
-    hipLaunchKernelGGL(moe_stream_kernel<F32>, dim3(grid), dim3(512), 0, stream, p);
+    hipLaunchKernelGGL(moe_stream_kernel<F32>, dim3(grid), dim3(512), lds, stream, p);
   }
   return hipGetLastError();
+}
+
+hipError_t prepare_stream_kernel() {
+  const size_t max_lds = static_cast<size_t>(8) * ROUTER_LDS_FLOATS * sizeof(float);
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(moe_stream_kernel<BF16>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     static_cast<int>(max_lds));
+  if (e != hipSuccess) return e;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(moe_stream_kernel<F32>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                             static_cast<int>(max_lds));
 }
 
 }  // namespace fmoe

@@ -154,5 +154,21 @@ class MoeKernelLauncher:
     def set_wait_limit_ms(self, ms):
         _hip_check(self._lib.flashMoeSetWaitLimitMs(self._h, float(ms)), "flashMoeSetWaitLimitMs")
 
+    TRACE_DTYPE = np.dtype([("ticket", "<u4"), ("kind", "<u4"), ("worker", "<u4"), ("aux", "<u4"),
+                            ("t_fetch", "<i8"), ("t_ready", "<i8"), ("t_end", "<i8"),
+                            ("pad", "<i8")])
+
+    def trace_enable(self, capacity):
+        _hip_check(self._lib.flashMoeTraceEnable(self._h, int(capacity)), "flashMoeTraceEnable")
+        self._trace_cap = int(capacity)
+
+    def trace_read(self):
+        """Records of the traced launches since the last read (numpy structured array)."""
+        rec = np.empty(self._trace_cap, self.TRACE_DTYPE)
+        with torch.cuda.device(self._device):
+            _hip_check(self._lib.flashMoeTraceRead(self._h, rec.ctypes.data, self._trace_cap,
+                                                   _stream()), "flashMoeTraceRead")
+        return rec[rec["kind"] != 0xFFFFFFFF]
+
     def sched_for(self, tokens_num):
         return self._lib.flashMoeSchedFor(self._h, int(tokens_num))

@@ -94,6 +94,19 @@ int flashMoeStatus(FlashMoeLauncher* l, unsigned* error_bits, unsigned* launches
  * (default 2000). A wait that runs out raises error bit 1 and ends the launch. */
 int flashMoeSetWaitLimitMs(FlashMoeLauncher* l, double ms);
 
+/* Task timeline for profiling (no counterpart in the reference, whose only
+ * timing aid is the host-side hipEvent helper of
+ * test/singleGPU/cpp/benchmarks/benchmarkUtils.h:26-52). Enable allocates
+ * `capacity` 48-byte records (0 frees them and turns tracing off); a traced
+ * launch writes one record per task, indexed by ticket:
+ *   { u32 ticket, kind, worker, aux; i64 t_fetch, t_ready, t_end, pad }
+ * kind: 0 router dot, 1 scan, 2 scatter, 3 gate/up, 4 down, 5 combine, 6 router
+ * select; times in
+ * ticks of the 100 MHz device wall clock. Read waits for `stream`, copies up to
+ * max_records records to the host and marks all records unused (all bits set). */
+int flashMoeTraceEnable(FlashMoeLauncher* l, unsigned capacity);
+int flashMoeTraceRead(FlashMoeLauncher* l, void* records, unsigned max_records, void* stream);
+
 /* Which scheduling variant a launch of tokens_num tokens would use. */
 int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num);
 
