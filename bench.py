@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused MoE layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME]
+
+A "step" is one forward pass of the layer over one batch of synthetic tokens
+(inputs already resident in HBM). The default workload is the Qwen3-30B-A3B
+decode batch (T=64). Prints ONE JSON line with the whole-job throughput, the
+roofline position of the (single) kernel of a step, measured with events on the
+launch stream, and the CPU oracle timed on this host beside it.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+MFMA_F32_PEAK_TFLOPS = 157.3
+
+# which roofline bounds each workload
+BOUND = {
+    "tiny_f32": "hbm",
+    "qwen3_30b_decode": "hbm",
+    "qwen3_30b_prefill": "mfma",
+    "qwen3_235b_t256": "hbm",
+    "qwen3_235b_t4096": "hbm",
+    "qwen3_30b_imbalance": "mfma",
+}
+
+
+def algorithmic_bytes(cfg, active_experts):
+    """Weights of the experts actually selected once, router weight once,
+    activations in and out once (no scratch traffic)."""
+    b = 2 if cfg.dtype == "bf16" else 4
+    return (active_experts * 3 * cfg.H * cfg.I + cfg.E * cfg.H + 2 * cfg.T * cfg.H) * b
+
+
+def algorithmic_flops(cfg):
+    return cfg.T * cfg.k * 6 * cfg.H * cfg.I + 2 * cfg.T * cfg.H * cfg.E
+
+
+def cpu_baseline(cfg, inp, seconds_budget=25.0):
+    """The CPU oracle (restatement of the reference's CPU MoE, one thread, as the
+    reference ships it) on a bounded sample of the same workload."""
+    from oracle import oracle
+
+    gate = inp["gate"].float().cpu().numpy()
+    ffn1 = inp["ffn1"].float().cpu().numpy()
+    ffn2 = inp["ffn2"].float().cpu().numpy()
+    bias = None if inp["bias"] is None else inp["bias"].float().cpu().numpy()
+    x = inp["tokens"].float().cpu().numpy()
+    # cost is linear in tokens: time 2 tokens, then size the sample to the budget
+    t0 = time.perf_counter()
+    oracle.forward(x[:2], gate, ffn1, ffn2, cfg.k, bias=bias, nthreads=1)
+    per_tok = (time.perf_counter() - t0) / 2
+    n = int(max(2, min(cfg.T, seconds_budget / max(per_tok, 1e-9))))
+    # repeat the sample until about 10 s of CPU work have been timed
+    reps = int(max(1, min(50, 10.0 / max(per_tok * n, 1e-9))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        oracle.forward(x[:n], gate, ffn1, ffn2, cfg.k, bias=bias, nthreads=1)
+    dt = (time.perf_counter() - t0) / reps
+    return {
+        "value": n / dt,
+        "unit": "tokens/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": "first %d of %d tokens of the workload, %d passes of %.2f s, one thread"
+                  % (n, cfg.T, reps, dt),
+        "us_per_layer_extrapolated": dt / n * cfg.T * 1e6,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="qwen3_30b_decode")
+    ap.add_argument("--seed", type=int, default=7907)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sched", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs the MoE layer on ONE GPU (no collectives, no "
+                 "multi-GPU path); run with --gpus 1")
+
+    import torch
+
+    from flash_distributed_moe_amd import synth
+    from flash_distributed_moe_amd.flashMoeLauncher import MoeKernelLauncher
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    cfg = synth.CONFIGS[args.config]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    inp = synth.make_inputs_torch(cfg, args.seed, dev)
+    x = inp["tokens"]
+    out = torch.empty_like(x)
+
+    launcher = MoeKernelLauncher()
+    launcher.create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T,
+                    launcher.getDistributedUniqueId(empty=True), 0, 1, top_k=cfg.k,
+                    router_bias=inp["bias"], sched=args.sched)
+
+    for _ in range(args.warmup):
+        launcher.launch(x, out)
+    torch.cuda.synchronize()
+
+    # whole-job wall time over exactly K steps
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        launcher.launch(x, out)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    # per-launch kernel duration: events on the launch stream around single launches
+    n_ev = min(args.steps, 200)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+           for _ in range(n_ev)]
+    for a, b in evs:
+        a.record()
+        launcher.launch(x, out)
+        b.record()
+    torch.cuda.synchronize()
+    durs = sorted(a.elapsed_time(b) for a, b in evs)  # ms
+    kernel_ms_avg = sum(durs) / len(durs)
+    kernel_ms_med = durs[len(durs) // 2]
+
+    err, _ = launcher.status()
+    if err:
+        sys.exit("bench.py: device error bits %d" % err)
+    routing = launcher.routing(cfg.T)
+    active = int((routing["counts"] > 0).sum())
+
+    bound = BOUND.get(cfg.name, "hbm")
+    abytes = algorithmic_bytes(cfg, active)
+    aflops = algorithmic_flops(cfg)
+    if bound == "hbm":
+        achieved = abytes / (kernel_ms_avg * 1e-3) / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = aflops / (kernel_ms_avg * 1e-3) / 1e12
+        peak = MFMA_BF16_PEAK_TFLOPS if cfg.dtype == "bf16" else MFMA_F32_PEAK_TFLOPS
+        unit = "TFLOP/s"
+    roofline = {
+        "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
+        "frac": achieved / peak, "traffic": None,
+        "kernel": "moe_stream_kernel" if launcher.sched_for(cfg.T) == 1 else "moe_tiled_kernel",
+        "kernel_us_avg": kernel_ms_avg * 1e3, "kernel_us_median": kernel_ms_med * 1e3,
+        "algorithmic_bytes": abytes, "algorithmic_flops": aflops, "active_experts": active,
+        "hbm_frac": abytes / (kernel_ms_avg * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "mfma_frac": aflops / (kernel_ms_avg * 1e-3) / 1e12 /
+        (MFMA_BF16_PEAK_TFLOPS if cfg.dtype == "bf16" else MFMA_F32_PEAK_TFLOPS),
+    }
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(cfg, inp)
+    launcher.destroy()
+
+    line = {
+        "metric": "MoE-layer tokens/s (Qwen3-style fused MoE forward, us/layer alongside)",
+        "value": cfg.T / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "us_per_layer": ms_per_step * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": cfg.dtype,
+        "data": "synthetic (seeded Irwin-Hall normal weights sigma 0.02, activations sigma 1)",
+        "config": {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E,
+                   "top_k": cfg.k, "intermediate": cfg.I, "hot_experts": cfg.hot,
+                   "seed": args.seed},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

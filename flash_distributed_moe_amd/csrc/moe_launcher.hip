@@ -34,6 +34,7 @@ hipError_t prepare_stream_kernel();
     if (fmoe_err_ != hipSuccess) {                                         \
       printf("[MOE HIP ERROR: %s:%i]: %s\n", FMOE_FILENAME, __LINE__,      \
              hipGetErrorString(fmoe_err_));                                \
+      fflush(stdout);                                                      \
       return fmoe_err_;                                                    \
     }                                                                      \
   } while (0)
@@ -41,6 +42,7 @@ hipError_t prepare_stream_kernel();
 #define FMOE_FAIL(code, fmt, ...)                                                      \
   do {                                                                                 \
     printf("[MOE ERROR: %s:%i]: " fmt "\n", FMOE_FILENAME, __LINE__, ##__VA_ARGS__);   \
+    fflush(stdout);                                                                    \
     return (code);                                                                     \
   } while (0)
 
