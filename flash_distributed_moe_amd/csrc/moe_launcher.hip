@@ -22,6 +22,9 @@
 namespace fmoe {
 hipError_t launch_stream_kernel(const Params& p, int dtype, int grid, hipStream_t stream);
 hipError_t prepare_stream_kernel();
+hipError_t launch_tiled_kernel(const Params& p, int grid, hipStream_t stream);
+hipError_t prepare_tiled_kernel();
+int tiled_max_tokens();
 }
 
 #define FMOE_FILENAME (strrchr(__FILE__, '/') ? strrchr(__FILE__, '/') + 1 : __FILE__)
@@ -227,8 +230,8 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
       khz > 0)
     l->ticks_per_ms = khz;
   l->spin_limit = 2000 * l->ticks_per_ms;
-  if ((e = fmoe::prepare_stream_kernel()) != hipSuccess)
-    return fail(e);
+  if ((e = fmoe::prepare_stream_kernel()) != hipSuccess) return fail(e);
+  if ((e = fmoe::prepare_tiled_kernel()) != hipSuccess) return fail(e);
   if ((e = hipMalloc(reinterpret_cast<void**>(&l->ws), l->layout.total)) != hipSuccess)
     return fail(e);
   if ((e = hipMemsetAsync(l->ws, 0, l->layout.zero_bytes, stream)) != hipSuccess) return fail(e);
@@ -237,10 +240,21 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
   return hipSuccess;
 }
 
+// The tiled variant needs bf16, tile-aligned shapes and a batch its scan tables
+// can hold; AUTO takes it once an expert sees about 48 rows on average.
+static bool tiled_eligible(const FlashMoeLayerDesc& d, int tokens_num) {
+  return d.dtype == FLASH_MOE_BF16 && d.hidden % 256 == 0 && d.intermediate % 128 == 0 &&
+         tokens_num <= fmoe::tiled_max_tokens();
+}
+
 int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num) {
-  (void)tokens_num;
   if (l == nullptr) return -1;
-  return FLASH_MOE_SCHED_STREAM;
+  const FlashMoeLayerDesc& d = l->desc;
+  if (d.sched == FLASH_MOE_SCHED_STREAM) return FLASH_MOE_SCHED_STREAM;
+  if (!tiled_eligible(d, tokens_num)) return FLASH_MOE_SCHED_STREAM;
+  if (d.sched == FLASH_MOE_SCHED_TILED) return FLASH_MOE_SCHED_TILED;
+  const long long rows = static_cast<long long>(tokens_num) * d.top_k;
+  return rows >= 48ll * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
 }
 
 int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int tokens_num,
@@ -256,7 +270,11 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
     FMOE_FAIL(hipErrorInvalidValue, "null tokens/output pointer");
   const fmoe::Params p = make_params(l, tokens, output, tokens_num);
   l->last_tokens = tokens_num;
-  FMOE_HIP_CHECK(fmoe::launch_stream_kernel(p, l->desc.dtype, p.n_groups, stream));
+  if (flashMoeSchedFor(l, tokens_num) == FLASH_MOE_SCHED_TILED) {
+    FMOE_HIP_CHECK(fmoe::launch_tiled_kernel(p, p.n_groups, stream));
+  } else {
+    FMOE_HIP_CHECK(fmoe::launch_stream_kernel(p, l->desc.dtype, p.n_groups, stream));
+  }
   return hipSuccess;
 }
 

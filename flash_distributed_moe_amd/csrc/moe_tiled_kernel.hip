@@ -1,0 +1,674 @@
+// Persistent MoE kernel, tiled ("fat") variant for gfx950: the shape for
+// batches where an expert sees hundreds of rows (prefill) and the layer is
+// bound by MFMA throughput, bf16 only.
+//
+// One workgroup of 4 waves per CU draws workgroup-wide task tickets from the
+// same kind of counter as the streaming variant; tasks depend only on tasks
+// with smaller tickets. Stages (ticket order):
+//   router   32 tokens x all experts: logits in the oracle's summation order on
+//            the vector ALUs (a 4x4 register tile of sequential chains per
+//            thread, operands staged transposed in LDS), then top-k / softmax
+//   scan     per-expert counts, offsets, 256-row tile table
+//   scatter  32 tokens: permuted row of every (token, slot)
+//   gate/up  (row tile, 128 h columns): 256x256x64 MFMA tile, gate and up
+//            columns side by side so that SiLU(gate)*up happens in registers
+//   down     (row tile, 256 output columns): same tile, weighted rows to y
+//   combine  8 tokens: out = sum over slots of y
+// GEMM tile: 256 token rows x 256 weight rows, K stepped by 64 through
+// double-buffered LDS (rows padded to 144 bytes so 8 consecutive rows hit
+// different banks); each wave owns 128x128 of it as 4x4 MFMA 32x32x16 blocks,
+// 256 accumulator registers. Weight rows are the MFMA "A" operand so that a
+// lane ends up with runs of 4 consecutive output columns of one token row.
+//
+// Replaces, for this regime, the reference's moeKernel
+// (src/hip/kernel/moeKernel.h:37-107) and its TILE_M=1 GEMV tiles
+// (src/hip/kernel/tasks/internal/gemmImpl/basicGemmTileImpl.h:14-94).
+#include "moe_device.h"
+
+namespace fmoe {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int TM = 256;            // token rows per tile
+constexpr int TN = 256;            // weight rows per tile
+constexpr int TK = 64;             // k per LDS stage
+constexpr int TLD = TK + 8;        // LDS row stride, bf16 elements (144 bytes)
+constexpr int T_THREADS = 256;
+constexpr int G1_COLS = TN / 2;    // h columns per gate/up task
+constexpr int RT_TOK = 32;         // tokens per router / scatter task
+constexpr int RT_KC = 64;          // router k-chunk
+constexpr int RT_XLD = RT_TOK + 4;     // floats per k-row of the transposed token chunk
+constexpr int RT_WLD = 128 + 4;        // floats per k-row of the transposed expert chunk
+constexpr int CMB_TOK = 8;         // tokens per combine task
+
+constexpr int TILE_LDS_BYTES = 2 * (TM + TN) * TLD * 2;  // 147456
+constexpr int ROUTER_LDS_BYTES = RT_KC * (RT_XLD + RT_WLD) * 4 + RT_TOK * MAX_EXPERTS * 8 +
+                                 4 * SELECT_LDS_BYTES;
+constexpr int TILED_LDS_BYTES = TILE_LDS_BYTES > ROUTER_LDS_BYTES ? TILE_LDS_BYTES : ROUTER_LDS_BYTES;
+
+extern __shared__ __align__(16) unsigned char lds_raw[];
+
+// ---------------------------------------------------------- workgroup helpers
+struct WgShared {  // small static LDS block
+  unsigned ticket;
+  unsigned ok;
+  unsigned flag[4];
+};
+
+// Thread 0 waits (bounded) for *p >= target; every thread learns the outcome.
+__device__ __forceinline__ bool wg_wait_ge(const Params& p, const unsigned* ptr, unsigned target,
+                                           WgShared* sh) {
+  if (threadIdx.x == 0) {
+    unsigned ok = 1u;
+    if (ld_relaxed(ptr) < target) {
+      const long long t0 = wall_clock64();
+      unsigned spins = 0;
+      while (ld_relaxed(ptr) < target) {
+        if ((++spins & 31u) == 0u && ld_relaxed(&p.ctl->error.v) != 0u) {
+          ok = 0u;
+          break;
+        }
+        if (wall_clock64() - t0 > p.spin_limit) {
+          or_relaxed(&p.ctl->error.v, ERR_TIMEOUT);
+          ok = 0u;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(16);
+      }
+    }
+    sh->ok = ok;
+  }
+  __syncthreads();
+  const bool ok = sh->ok != 0u;
+  __syncthreads();
+  fence_acquire();
+  return ok;
+}
+
+__device__ __forceinline__ bool wg_wait_flag(const Params& p, int which, WgShared* sh) {
+  if (sh->flag[which] != 0u) return true;  // seen before by this workgroup
+  const bool ok = wg_wait_ge(p, &p.wgflags[blockIdx.x].f[which], 1u, sh);
+  if (ok && threadIdx.x == 0) sh->flag[which] = 1u;
+  __syncthreads();
+  return ok;
+}
+
+// All threads' coherent stores have completed, then one thread bumps the counter.
+__device__ __forceinline__ unsigned wg_arrive(unsigned* counter, WgShared* sh) {
+  fence_release();
+  __syncthreads();
+  if (threadIdx.x == 0) sh->ticket = add_relaxed(counter, 1u);
+  __syncthreads();
+  const unsigned old = sh->ticket;
+  __syncthreads();
+  return old;
+}
+
+__device__ __forceinline__ void wg_broadcast_flag(const Params& p, int which) {
+  const int n = p.n_groups;
+  WgFlags* flags = p.wgflags;
+  for (int g = threadIdx.x; g < n; g += blockDim.x) st_relaxed(&flags[g].f[which], 1u);
+}
+
+// --------------------------------------------------------------------- router
+// Logits as in test/singleGPU/cpp/moe/reference/refGemm.h:21-24 (one chain per
+// output, k ascending; bf16 products are exact in float so fma == mul+add),
+// then selection as in refTopk.h:36-58 / refMoeGate.h:27-30.
+__device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
+  const int T = p.T, E = p.E, H = p.H;
+  const unsigned short* tokens = reinterpret_cast<const unsigned short*>(p.tokens);
+  const unsigned short* gate = reinterpret_cast<const unsigned short*>(p.gate);
+  float* xT = reinterpret_cast<float*>(lds_raw);   // [RT_KC][RT_XLD]
+  float* wT = xT + RT_KC * RT_XLD;                 // [RT_KC][RT_WLD]
+  unsigned long long* keys = reinterpret_cast<unsigned long long*>(wT + RT_KC * RT_WLD);
+  unsigned long long* sel = keys + RT_TOK * MAX_EXPERTS;  // 4 waves x SELECT_LDS_BYTES
+  const int tid = threadIdx.x;
+  const int tt = tid >> 5, te = tid & 31;          // 4 tokens x 4 experts per thread
+  const int t0 = blk * RT_TOK;
+
+  for (int e0 = 0; e0 < E; e0 += 128) {
+    float acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) acc[a][b] = 0.0f;
+
+    // staging map: one token chunk and four expert chunks of 16 bytes per thread
+    const int xr = tid & 31, xc = tid >> 5;
+    const unsigned short* xsrc =
+        tokens + static_cast<size_t>(min(t0 + xr, T - 1)) * H + xc * 8;
+    const unsigned short* wsrc[4];
+    int wr[4], wc[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int c = tid + 256 * q;
+      wr[q] = c & 127;
+      wc[q] = c >> 7;
+      wsrc[q] = gate + static_cast<size_t>(min(e0 + wr[q], E - 1)) * H + wc[q] * 8;
+    }
+    uint4 xv = ld16(xsrc);
+    uint4 wv[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) wv[q] = ld16(wsrc[q]);
+
+    for (int k0 = 0; k0 < H; k0 += RT_KC) {
+      __syncthreads();  // previous chunk fully consumed
+      {
+        float f[8];
+        unpack<BF16>(xv, f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xT[(xc * 8 + i) * RT_XLD + xr] = f[i];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          unpack<BF16>(wv[q], f);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) wT[(wc[q] * 8 + i) * RT_WLD + wr[q]] = f[i];
+        }
+      }
+      __syncthreads();
+      if (k0 + RT_KC < H) {
+        xv = ld16(xsrc + k0 + RT_KC);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) wv[q] = ld16(wsrc[q] + k0 + RT_KC);
+      }
+#pragma unroll 8
+      for (int k = 0; k < RT_KC; ++k) {
+        const float4 x4 = *reinterpret_cast<const float4*>(xT + k * RT_XLD + tt * 4);
+        const float4 w4 = *reinterpret_cast<const float4*>(wT + k * RT_WLD + te * 4);
+        const float xa[4] = {x4.x, x4.y, x4.z, x4.w};
+        const float wa[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int b = 0; b < 4; ++b) acc[a][b] = __builtin_fmaf(xa[a], wa[b], acc[a][b]);
+      }
+    }
+    // keys of this expert slab into LDS: keys[token][expert]
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int e = e0 + te * 4 + b;
+        float v = acc[a][b];
+        if (p.bias != nullptr && e < E) v = __fadd_rn(v, as_global(p.bias)[e]);
+        if (e < MAX_EXPERTS) keys[(tt * 4 + a) * MAX_EXPERTS + e] = make_key(v, e, e < E);
+      }
+  }
+  __syncthreads();
+  // selection: each wave takes 8 of the 32 tokens
+  const int wave = tid >> 6, lane = tid & 63;
+  unsigned long long* lk = sel + wave * (SELECT_LDS_BYTES / 8);
+  for (int i = 0; i < RT_TOK / 4; ++i) {
+    const int tl = wave * (RT_TOK / 4) + i;
+    const int t = t0 + tl;
+    if (t < T) {
+      unsigned long long key[MAX_EXPERTS / 64];
+#pragma unroll
+      for (int j = 0; j < MAX_EXPERTS / 64; ++j) {
+        const int e = lane + 64 * j;
+        key[j] = e < E ? keys[tl * MAX_EXPERTS + e] : 0ull;
+      }
+      router_select(p, t, key, lk);
+    }
+  }
+}
+
+// ----------------------------------------------------------------------- scan
+// Same tables as the streaming variant's scan, computed by one workgroup:
+// thread e walks expert e's mask words (their popcounts were gathered into LDS
+// by all threads first), then one wave scans over the experts.
+__device__ __noinline__ void tiled_scan_task(const Params& p) {
+  const RouteTables r = route_tables(p);
+  const int tid = threadIdx.x;
+  const int wact = (r.T + 63) >> 6;
+  unsigned char* pc = lds_raw;                                       // [E][wact] popcounts
+  int* cnt = reinterpret_cast<int*>(lds_raw + ((MAX_EXPERTS * wact + 15) & ~15));  // [E]
+  const int total = r.E * wact;
+  for (int i0 = tid; i0 < total; i0 += T_THREADS * 8) {
+    unsigned long long m[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const int i = i0 + b * T_THREADS;
+      m[b] = 0ull;
+      if (i < total) m[b] = ldc(&r.masks[static_cast<size_t>(i / wact) * r.W + (i % wact)]);
+    }
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const int i = i0 + b * T_THREADS;
+      if (i < total) pc[i] = static_cast<unsigned char>(__popcll(m[b]));
+    }
+  }
+  __syncthreads();
+  if (tid < r.E) {
+    int c = 0;
+    int* wp = r.word_prefix + static_cast<size_t>(tid) * r.W;
+    for (int w = 0; w < wact; ++w) {
+      stc(&wp[w], c);
+      c += pc[tid * wact + w];
+    }
+    cnt[tid] = c;
+  }
+  __syncthreads();
+  if (tid < 64) {
+    const int lane = tid;
+    const int epl = (r.E + 63) >> 6;
+    int base = 0, tile_base = 0;
+    for (int j = 0; j < epl; ++j) {
+      const int e = lane + 64 * j;
+      const int c = e < r.E ? cnt[e] : 0;
+      const int incl = wave_inclusive_scan(c);
+      const int off = base + incl - c;
+      const int nt = (c + TM - 1) / TM;
+      const int tincl = wave_inclusive_scan(nt);
+      const int toff = tile_base + tincl - nt;
+      if (e < r.E) {
+        stc(&r.expert_count[e], c);
+        stc(&r.expert_offset[e], off);
+        for (int i = 0; i < nt; ++i) {
+          if (toff + i < r.max_mtiles) {
+            stc16(&r.mtiles[toff + i],
+                  make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + i * TM),
+                             static_cast<unsigned>(min(TM, c - i * TM)), 0u));
+          }
+        }
+      }
+      base += __shfl(incl, 63, 64);
+      tile_base += __shfl(tincl, 63, 64);
+    }
+    if (lane == 0) {
+      stc(&r.expert_offset[r.E], base);
+      if (tile_base > r.max_mtiles) {
+        or_relaxed(&p.ctl->error.v, ERR_CAPACITY);
+        tile_base = 0;
+      }
+      stc(&p.ctl->n_mtiles.v, static_cast<unsigned>(tile_base));
+    }
+  }
+  fence_release();
+  __syncthreads();
+  wg_broadcast_flag(p, FLAG_SCAN);
+}
+
+__device__ void tiled_scatter_task(const Params& p, int blk) {
+  const RouteTables r = route_tables(p);
+  const int i0 = blk * RT_TOK * r.K;
+  const int n = min(RT_TOK * r.K, r.T * r.K - i0);
+  for (int i = threadIdx.x; i < n; i += T_THREADS) scatter_entry(r, i0 + i);
+}
+
+// -------------------------------------------------------------- the GEMM tile
+// Per-thread staging map. Each k-step a thread moves 8 chunks of 16 bytes of
+// each operand: chunk q covers stage row (tid/8 + 32*q), bytes (tid%8)*16 of
+// the row's 128-byte k-slice. Weight rows are regular (two bases: stage rows
+// 0..127 and 128..255); token rows are given per chunk (gathered rows).
+struct TileRows {
+  const unsigned short* w_lo;  // stage row tid/8, this thread's k-chunk
+  const unsigned short* w_hi;  // stage row 128 + tid/8
+  size_t w_step;               // elements between stage rows 32 apart
+  const unsigned short* tbase;
+  int trow[8];                 // source row of token-stage row tid/8 + 32*q
+  size_t tstride;              // elements per source row
+  int lds_off;                 // element offset of chunk 0 inside one operand stage
+};
+
+__device__ __forceinline__ f32x16 mma32(const uint4& a, const uint4& b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// acc[i][j] (+)= W-block i (32 weight rows) x token-block j (32 token rows).
+// wblk[i]: first weight row of block i inside the weight stage; tokens of this
+// wave start at tok0. jmax: token blocks of this wave that hold valid rows.
+// COH_T: the token operand was written by other workers during this launch.
+template <bool COH_T>
+__device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, const int (&wblk)[4],
+                                          int tok0, int jmax, f32x16 (&acc)[4][4]) {
+  unsigned short* wst = reinterpret_cast<unsigned short*>(lds_raw);          // [2][TN][TLD]
+  unsigned short* tst = wst + 2 * TN * TLD;                                  // [2][TM][TLD]
+  const int lane = threadIdx.x & 63;
+  const int r32 = lane & 31, kq = lane >> 5;
+
+  uint4 wreg[8], treg[8];
+  auto issue = [&](int ks) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      wreg[q] = ld16(rows.w_lo + q * rows.w_step + ks * TK);
+      wreg[q + 4] = ld16(rows.w_hi + q * rows.w_step + ks * TK);
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const unsigned short* src = rows.tbase + static_cast<size_t>(rows.trow[q]) * rows.tstride + ks * TK;
+      treg[q] = COH_T ? ldc16(src) : ld16(src);
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      *reinterpret_cast<uint4*>(wst + buf * TN * TLD + rows.lds_off + q * 32 * TLD) = wreg[q];
+      *reinterpret_cast<uint4*>(tst + buf * TM * TLD + rows.lds_off + q * 32 * TLD) = treg[q];
+    }
+  };
+
+  issue(0);
+  stash(0);
+  __syncthreads();
+  for (int ks = 0; ks < ksteps; ++ks) {
+    const int buf = ks & 1;
+    if (ks + 1 < ksteps) issue(ks + 1);
+    const unsigned short* wb = wst + buf * TN * TLD;
+    const unsigned short* tb = tst + buf * TM * TLD;
+#pragma unroll
+    for (int kk = 0; kk < TK / 16; ++kk) {
+      uint4 a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        a[i] = *reinterpret_cast<const uint4*>(wb + (wblk[i] + r32) * TLD + kk * 16 + kq * 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (j < jmax)
+          b[j] = *reinterpret_cast<const uint4*>(tb + (tok0 + j * 32 + r32) * TLD + kk * 16 + kq * 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (j < jmax) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i][j] = mma32(a[i], b[j], acc[i][j]);
+        }
+    }
+    if (ks + 1 < ksteps) stash(buf ^ 1);
+    __syncthreads();
+  }
+}
+
+// gate/up: h[row, n0 .. n0+128) for one row tile
+// (test/singleGPU/cpp/moe/reference/refExpertFFN1.h:51-65).
+__device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& tile, int nblk) {
+  const int H = p.H, I = p.I, K = p.K;
+  const int n0 = nblk * G1_COLS;
+  const unsigned short* w13 =
+      reinterpret_cast<const unsigned short*>(p.ffn1) + static_cast<size_t>(tile.expert) * 2 * I * H;
+  const int srow = threadIdx.x >> 3, kc = threadIdx.x & 7;
+  TileRows rows;
+  // weight stage rows 0..127: gate rows n0+row, 128..255: up rows I+n0+(row-128)
+  rows.w_lo = w13 + static_cast<size_t>(n0 + srow) * H + kc * 8;
+  rows.w_hi = w13 + static_cast<size_t>(I + n0 + srow) * H + kc * 8;
+  rows.w_step = static_cast<size_t>(32) * H;
+  rows.tbase = reinterpret_cast<const unsigned short*>(p.tokens) + kc * 8;
+  rows.tstride = static_cast<size_t>(H);
+  rows.lds_off = srow * TLD + kc * 8;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const int tr = min(srow + 32 * q, tile.rows - 1);
+    rows.trow[q] = ldc(&p.perm[tile.row0 + tr]) / K;
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wn = wave & 1, wm = wave >> 1;
+  const int wblk[4] = {wn * 64, wn * 64 + 32, G1_COLS + wn * 64, G1_COLS + wn * 64 + 32};
+  const int tok0 = wm * 128;
+  const int jmax = min(4, max(0, (tile.rows - tok0 + 31) / 32));
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  tile_gemm<false>(rows, H / TK, wblk, tok0, jmax, acc);
+
+  const int r32 = lane & 31, kq = lane >> 5;
+  unsigned short* h = reinterpret_cast<unsigned short*>(p.h);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int trow = tok0 + j * 32 + r32;
+    if (j < jmax && trow < tile.rows) {
+      unsigned short* hrow = h + static_cast<size_t>(tile.row0 + trow) * I + n0 + wn * 64;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          float hv[4];
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            hv[v] = silu_mul(acc[i][j][g4 * 4 + v], acc[i + 2][j][g4 * 4 + v]);
+          const unsigned lo = f2bf(hv[0]) | (f2bf(hv[1]) << 16);
+          const unsigned hi = f2bf(hv[2]) | (f2bf(hv[3]) << 16);
+          stc(reinterpret_cast<unsigned long long*>(hrow + i * 32 + g4 * 8 + kq * 4),
+              static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32));
+        }
+    }
+  }
+}
+
+// down: y[t*K+slot, n0 .. n0+256) = w * (h[row] . W2[e]^T)
+// (refFullMoe.h:58-65, src/hip/kernel/tasks/ffn2Task.h:37-40).
+__device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& tile, int nblk) {
+  const int H = p.H, I = p.I;
+  const int n0 = nblk * TN;
+  const unsigned short* w2 =
+      reinterpret_cast<const unsigned short*>(p.ffn2) + static_cast<size_t>(tile.expert) * H * I;
+  const int srow = threadIdx.x >> 3, kc = threadIdx.x & 7;
+  TileRows rows;
+  rows.w_lo = w2 + static_cast<size_t>(n0 + srow) * I + kc * 8;
+  rows.w_hi = w2 + static_cast<size_t>(n0 + 128 + srow) * I + kc * 8;
+  rows.w_step = static_cast<size_t>(32) * I;
+  rows.tbase = reinterpret_cast<const unsigned short*>(p.h) + kc * 8;
+  rows.tstride = static_cast<size_t>(I);
+  rows.lds_off = srow * TLD + kc * 8;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) rows.trow[q] = tile.row0 + min(srow + 32 * q, tile.rows - 1);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wn = wave & 1, wm = wave >> 1;
+  const int wblk[4] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
+  const int tok0 = wm * 128;
+  const int jmax = min(4, max(0, (tile.rows - tok0 + 31) / 32));
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  tile_gemm<true>(rows, I / TK, wblk, tok0, jmax, acc);
+
+  const int r32 = lane & 31, kq = lane >> 5;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int trow = tok0 + j * 32 + r32;
+    if (j < jmax && trow < tile.rows) {
+      const float w = ldc(&p.row_w[tile.row0 + trow]);
+      float* yrow = p.y + static_cast<size_t>(ldc(&p.perm[tile.row0 + trow])) * H + n0 + wn * 128;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          stc16(yrow + i * 32 + g4 * 8 + kq * 4,
+                make_uint4(__float_as_uint(acc[i][j][g4 * 4 + 0] * w),
+                           __float_as_uint(acc[i][j][g4 * 4 + 1] * w),
+                           __float_as_uint(acc[i][j][g4 * 4 + 2] * w),
+                           __float_as_uint(acc[i][j][g4 * 4 + 3] * w)));
+        }
+    }
+  }
+}
+
+// combine: out[t] = sum over slots, in slot order, of y[t*K+slot]
+// (refFullMoe.h:35,62-65).
+__device__ __noinline__ void tiled_combine_task(const Params& p, int blk) {
+  const int H = p.H, K = p.K, T = p.T;
+  unsigned short* out = reinterpret_cast<unsigned short*>(p.out);
+  for (int tl = 0; tl < CMB_TOK; ++tl) {
+    const int t = blk * CMB_TOK + tl;
+    if (t >= T) break;
+    for (int c = threadIdx.x * 4; c < H; c += T_THREADS * 4) {
+      float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int k = 0; k < K; ++k) {
+        if (ldc(&p.topk_idx[static_cast<size_t>(t) * K + k]) < 0) continue;
+        const uint4 v = ldc16(p.y + (static_cast<size_t>(t) * K + k) * H + c);
+        s.x += __uint_as_float(v.x);
+        s.y += __uint_as_float(v.y);
+        s.z += __uint_as_float(v.z);
+        s.w += __uint_as_float(v.w);
+      }
+      const unsigned lo = f2bf(s.x) | (f2bf(s.y) << 16);
+      const unsigned hi = f2bf(s.z) | (f2bf(s.w) << 16);
+      *as_global(reinterpret_cast<unsigned long long*>(out + static_cast<size_t>(t) * H + c)) =
+          static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32);
+    }
+    if ((t & 63) == 0) {
+      for (int e = threadIdx.x; e < p.E; e += T_THREADS)
+        stc(&p.masks[static_cast<size_t>(e) * p.W + (t >> 6)], 0ull);
+    }
+  }
+}
+
+// ---------------------------------------------------------------- worker loop
+__global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
+  __shared__ WgShared sh;
+  if (threadIdx.x == 0) {
+    sh.ticket = 0u;
+    sh.ok = 1u;
+    sh.flag[0] = sh.flag[1] = sh.flag[2] = sh.flag[3] = 0u;
+  }
+  __syncthreads();
+  Control* ctl = p.ctl;
+  const unsigned T = static_cast<unsigned>(p.T);
+  const unsigned n_rt = (T + RT_TOK - 1u) / RT_TOK;
+  const unsigned t_scan = n_rt;
+  const unsigned t_scatter0 = n_rt + 1u;
+  const unsigned t_dyn0 = t_scatter0 + n_rt;
+  const unsigned nt1 = static_cast<unsigned>(p.I / G1_COLS);
+  const unsigned nt2 = static_cast<unsigned>(p.H / TN);
+  const unsigned ncmb = (T + CMB_TOK - 1u) / CMB_TOK;
+  const unsigned n_groups = gridDim.x;
+  unsigned n1 = 0, n2 = 0;
+  bool have_dyn = false, first = true;
+
+  while (true) {
+    const long long t_fetch = p.trace ? wall_clock64() : 0;
+    if (threadIdx.x == 0) sh.ticket = first ? blockIdx.x : n_groups + add_relaxed(&ctl->ticket.v, 1u);
+    first = false;
+    __syncthreads();
+    const unsigned tk = sh.ticket;
+    __syncthreads();
+    unsigned kind = 0, aux = 0;
+    long long t_ready = 0;
+    bool ok = true;
+
+    if (tk < n_rt) {
+      kind = 0;
+      aux = tk;
+      if (p.trace) t_ready = wall_clock64();
+      tiled_router_task(p, static_cast<int>(tk));
+      wg_arrive(&ctl->router_done.v, &sh);
+    } else if (tk == t_scan) {
+      kind = 1;
+      ok = wg_wait_ge(p, &ctl->router_done.v, n_rt, &sh);
+      if (ok) {
+        if (p.trace) t_ready = wall_clock64();
+        tiled_scan_task(p);
+      }
+    } else if (tk < t_dyn0) {
+      kind = 2;
+      aux = tk - t_scatter0;
+      ok = wg_wait_flag(p, FLAG_SCAN, &sh);
+      if (ok) {
+        if (p.trace) t_ready = wall_clock64();
+        tiled_scatter_task(p, static_cast<int>(aux));
+        if (wg_arrive(&ctl->perm_done.v, &sh) == n_rt - 1u) wg_broadcast_flag(p, FLAG_PERM);
+      }
+    } else {
+      if (!have_dyn) {
+        ok = wg_wait_flag(p, FLAG_SCAN, &sh);
+        if (ok) {
+          const unsigned nm = ldc(&ctl->n_mtiles.v);
+          n1 = nm * nt1;
+          n2 = nm * nt2;
+          have_dyn = true;
+        }
+      }
+      const unsigned j = tk - t_dyn0;
+      if (!ok) {
+      } else if (j < n1) {
+        kind = 3;
+        aux = j / nt1;
+        ok = wg_wait_flag(p, FLAG_PERM, &sh);
+        if (ok) {
+          if (p.trace) t_ready = wall_clock64();
+          const TileDesc tile = ld_tile(&p.mtiles[aux]);
+          tiled_gateup_task(p, tile, static_cast<int>(j % nt1));
+          wg_arrive(&p.g1_done[aux].v, &sh);
+        }
+      } else if (j < n1 + n2) {
+        kind = 4;
+        aux = (j - n1) / nt2;
+        ok = wg_wait_ge(p, &p.g1_done[aux].v, nt1, &sh);
+        if (ok) {
+          if (p.trace) t_ready = wall_clock64();
+          const TileDesc tile = ld_tile(&p.mtiles[aux]);
+          tiled_down_task(p, tile, static_cast<int>((j - n1) % nt2));
+          if (wg_arrive(&ctl->g2_done.v, &sh) == n2 - 1u) wg_broadcast_flag(p, FLAG_G2);
+        }
+      } else if (j < n1 + n2 + ncmb) {
+        kind = 5;
+        aux = j - n1 - n2;
+        if (n2 != 0u) ok = wg_wait_flag(p, FLAG_G2, &sh);
+        if (ok) {
+          if (p.trace) t_ready = wall_clock64();
+          tiled_combine_task(p, static_cast<int>(aux));
+        }
+      } else {
+        break;
+      }
+    }
+    if (!ok) break;
+    if (p.trace && threadIdx.x == 0 && tk < p.trace_cap) {
+      const long long t_end = wall_clock64();
+      TraceRec* r = p.trace + tk;
+      st16(r, u32x4{tk, kind, blockIdx.x, aux});
+      st16(reinterpret_cast<char*>(r) + 16,
+           u32x4{static_cast<unsigned>(t_fetch), static_cast<unsigned>(t_fetch >> 32),
+                 static_cast<unsigned>(t_ready), static_cast<unsigned>(t_ready >> 32)});
+      st16(reinterpret_cast<char*>(r) + 32,
+           u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), 0u, 0u});
+    }
+  }
+
+  // The last workgroup out returns every counter to zero for the next launch.
+  __syncthreads();
+  if (threadIdx.x == 0) sh.ok = (add_relaxed(&ctl->exit_count.v, 1u) == n_groups - 1u) ? 1u : 0u;
+  __syncthreads();
+  if (sh.ok) {
+    const unsigned nm = min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
+    for (unsigned i = threadIdx.x; i < nm; i += T_THREADS) stc(&p.g1_done[i].v, 0u);
+    for (unsigned g = threadIdx.x; g < n_groups; g += T_THREADS) {
+      stc(&p.wgflags[g].f[FLAG_SCAN], 0u);
+      stc(&p.wgflags[g].f[FLAG_PERM], 0u);
+      stc(&p.wgflags[g].f[FLAG_G2], 0u);
+    }
+    if (threadIdx.x == 0) {
+      stc(&ctl->launches.v, ldc(&ctl->launches.v) + 1u);
+      stc(&ctl->router_done.v, 0u);
+      stc(&ctl->perm_done.v, 0u);
+      stc(&ctl->g2_done.v, 0u);
+      stc(&ctl->n_mtiles.v, 0u);
+      stc(&ctl->exit_count.v, 0u);
+      stc(&ctl->ticket.v, 0u);
+    }
+  }
+}
+
+// Largest token count the scan task's LDS tables allow.
+int tiled_max_tokens() { return ((TILED_LDS_BYTES - 2048) / MAX_EXPERTS) * 64; }
+
+hipError_t launch_tiled_kernel(const Params& p, int grid, hipStream_t stream) {
+  hipLaunchKernelGGL(moe_tiled_kernel, dim3(grid), dim3(T_THREADS), TILED_LDS_BYTES, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t prepare_tiled_kernel() {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(moe_tiled_kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, TILED_LDS_BYTES);
+}
+
+}  // namespace fmoe

@@ -100,3 +100,36 @@ def test_relaunch_and_smaller_batch():
         assert case.launcher.status() == (0, 3)
     finally:
         case.close()
+
+
+@pytest.mark.parametrize("shape", [
+    # T, H, E, k, I: the tiled (MFMA 32x32, LDS-staged) variant forced on small problems
+    (300, 256, 8, 2, 128),      # ragged last row tile (75 rows per expert on average)
+    (700, 512, 4, 2, 256),      # several 256-row tiles per expert, ragged tail
+    (64, 256, 200, 6, 128),     # E > 128: two expert slabs in the router; tiny tiles
+    (1, 256, 8, 2, 128),        # a single token
+])
+def test_tiled_variant_forced(shape):
+    T, H, E, k, I = shape
+    cfg = synth.MoeConfig("tiled", T, H, E, k, I, "bf16")
+    print("tiled forced", shape, flush=True)
+    case = GpuCase(cfg, seed=T + E, sched=_lib.SCHED_TILED)
+    try:
+        assert case.launcher.sched_for(T) == _lib.SCHED_TILED
+        x = case.inp["tokens"]
+        out = case.run()
+        case.check_routing(x, case.launcher.routing(T))
+        err = case.check_outputs(x, out)
+        print("  max rel err %.3e" % err, flush=True)
+        # the streaming variant on the same inputs agrees on routing bit for bit
+        other = GpuCase(cfg, seed=T + E, sched=_lib.SCHED_STREAM, inputs=case.inp)
+        try:
+            out2 = other.run()
+            r1, r2 = case.launcher.routing(T), other.launcher.routing(T)
+            assert np.array_equal(r1["topk_idx"], r2["topk_idx"])
+            assert np.array_equal(r1["perm"], r2["perm"])
+            assert torch.allclose(out.float(), out2.float(), rtol=2e-2, atol=1e-3)
+        finally:
+            other.close()
+    finally:
+        case.close()
