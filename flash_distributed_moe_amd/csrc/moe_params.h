@@ -42,6 +42,8 @@ struct Control {
   ControlLine n_mtiles;     // row tiles produced by the scan
   ControlLine error;        // sticky error bits
   ControlLine launches;     // completed launches (diagnostic)
+  ControlLine xq[8];        // tiled variant: per-XCD ticket counters of the GEMM tasks
+  ControlLine cticket;      // tiled variant: combine tickets
 };
 
 // Phase flags, one line per workgroup: the worker that completes a phase

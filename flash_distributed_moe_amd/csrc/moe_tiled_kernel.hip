@@ -93,11 +93,21 @@ __device__ __forceinline__ bool wg_wait_flag(const Params& p, int which, WgShare
   return ok;
 }
 
-// All threads' coherent stores have completed, then one thread bumps the counter.
+// All threads' stores have completed, then one thread bumps the counter.
+// WRITEBACK: the task wrote tile data (h, y) with ordinary cached stores, so the
+// XCD's L2 is written back to memory first (one agent-scope release per task and
+// workgroup is cheap; per wave task it is not, which is why the streaming
+// variant writes through instead). Readers of h and y use ordinary loads: every
+// cache line of them has a single writer and is not read before it is final,
+// so no reader can hold a stale copy.
+template <bool WRITEBACK>
 __device__ __forceinline__ unsigned wg_arrive(unsigned* counter, WgShared* sh) {
   fence_release();
   __syncthreads();
-  if (threadIdx.x == 0) sh->ticket = add_relaxed(counter, 1u);
+  if (threadIdx.x == 0) {
+    if (WRITEBACK) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    sh->ticket = add_relaxed(counter, 1u);
+  }
   __syncthreads();
   const unsigned old = sh->ticket;
   __syncthreads();
@@ -328,8 +338,14 @@ __device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, cons
   const int lane = threadIdx.x & 63;
   const int r32 = lane & 31, kq = lane >> 5;
 
-  uint4 wreg[8], treg[8];
-  auto issue = [&](int ks) {
+  // Two register sets: the loads of k-step ks+2 are issued while ks is computed
+  // and are only needed (to be written to LDS) at the end of ks+1, so they have
+  // two full compute phases to arrive.
+  uint4 wr0[8], tr0[8], wr1[8], tr1[8];
+  auto issue = [&](uint4(&wreg)[8], uint4(&treg)[8], int ks) {
+#ifdef FMOE_DBG_NO_GLOBAL  // timing experiment: only the first two k-steps touch memory
+    if (ks >= 2) return;
+#endif
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       wreg[q] = ld16(rows.w_lo + q * rows.w_step + ks * TK);
@@ -341,20 +357,14 @@ __device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, cons
       treg[q] = COH_T ? ldc16(src) : ld16(src);
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](const uint4(&wreg)[8], const uint4(&treg)[8], int buf) {
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       *reinterpret_cast<uint4*>(wst + buf * TN * TLD + rows.lds_off + q * 32 * TLD) = wreg[q];
       *reinterpret_cast<uint4*>(tst + buf * TM * TLD + rows.lds_off + q * 32 * TLD) = treg[q];
     }
   };
-
-  issue(0);
-  stash(0);
-  __syncthreads();
-  for (int ks = 0; ks < ksteps; ++ks) {
-    const int buf = ks & 1;
-    if (ks + 1 < ksteps) issue(ks + 1);
+  auto compute = [&](int buf) {
     const unsigned short* wb = wst + buf * TN * TLD;
     const unsigned short* tb = tst + buf * TM * TLD;
 #pragma unroll
@@ -371,10 +381,32 @@ __device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, cons
       for (int j = 0; j < 4; ++j)
         if (j < jmax) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[i][j] = mma32(a[i], b[j], acc[i][j]);
+          for (int i = 0; i < 4; ++i) {
+#ifdef FMOE_DBG_NO_MFMA  // timing experiment: consume the fragments without the matrix core
+            acc[i][j][0] += __uint_as_float(a[i].x ^ b[j].y);
+#else
+            acc[i][j] = mma32(a[i], b[j], acc[i][j]);
+#endif
+          }
         }
     }
-    if (ks + 1 < ksteps) stash(buf ^ 1);
+  };
+
+  issue(wr0, tr0, 0);
+  if (ksteps > 1) issue(wr1, tr1, 1);
+  stash(wr0, tr0, 0);
+  __syncthreads();
+  for (int ks = 0; ks < ksteps; ks += 2) {
+    // even step: LDS buffer 0 holds ks, set 1 holds ks+1 (in flight)
+    if (ks + 2 < ksteps) issue(wr0, tr0, ks + 2);
+    compute(0);
+    if (ks + 1 < ksteps) stash(wr1, tr1, 1);
+    __syncthreads();
+    if (ks + 1 >= ksteps) break;
+    // odd step: LDS buffer 1 holds ks+1, set 0 holds ks+2 (in flight)
+    if (ks + 3 < ksteps) issue(wr1, tr1, ks + 3);
+    compute(1);
+    if (ks + 2 < ksteps) stash(wr0, tr0, 0);
     __syncthreads();
   }
 }
@@ -415,13 +447,15 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
 
   tile_gemm<false>(rows, H / TK, wblk, tok0, jmax, acc);
 
+  // Epilogue through LDS (the stage buffers are free now): each wave turns its
+  // 32-token x 64-column blocks into full 128-byte row segments of h.
   const int r32 = lane & 31, kq = lane >> 5;
   unsigned short* h = reinterpret_cast<unsigned short*>(p.h);
+  constexpr int SLD = 64 + 8;  // slab row stride, bf16 elements
+  unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * 32 * SLD;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int trow = tok0 + j * 32 + r32;
-    if (j < jmax && trow < tile.rows) {
-      unsigned short* hrow = h + static_cast<size_t>(tile.row0 + trow) * I + n0 + wn * 64;
+    if (j < jmax) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -430,11 +464,22 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
 #pragma unroll
           for (int v = 0; v < 4; ++v)
             hv[v] = silu_mul(acc[i][j][g4 * 4 + v], acc[i + 2][j][g4 * 4 + v]);
-          const unsigned lo = f2bf(hv[0]) | (f2bf(hv[1]) << 16);
-          const unsigned hi = f2bf(hv[2]) | (f2bf(hv[3]) << 16);
-          stc(reinterpret_cast<unsigned long long*>(hrow + i * 32 + g4 * 8 + kq * 4),
-              static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32));
+          uint2 pk;
+          pk.x = f2bf(hv[0]) | (f2bf(hv[1]) << 16);
+          pk.y = f2bf(hv[2]) | (f2bf(hv[3]) << 16);
+          *reinterpret_cast<uint2*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) = pk;
         }
+      lds_wave_sync();
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int rr = it * 8 + (lane >> 3), cc = (lane & 7) * 8;
+        const int trow = tok0 + j * 32 + rr;
+        const uint4 v = *reinterpret_cast<const uint4*>(slab + rr * SLD + cc);
+        if (trow < tile.rows)
+          st16(h + static_cast<size_t>(tile.row0 + trow) * I + n0 + wn * 64 + cc,
+               u32x4{v.x, v.y, v.z, v.w});
+      }
+      lds_wave_sync();
     }
   }
 }
@@ -469,25 +514,40 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  tile_gemm<true>(rows, I / TK, wblk, tok0, jmax, acc);
+  tile_gemm<false>(rows, I / TK, wblk, tok0, jmax, acc);
 
+  // Epilogue through LDS: 32-token x 128-column blocks become 512-byte row
+  // segments of y, scaled by the row's gate weight, at the row's (token, slot).
   const int r32 = lane & 31, kq = lane >> 5;
+  constexpr int SLD = 128 + 4;  // slab row stride, floats
+  float* slab = reinterpret_cast<float*>(lds_raw) + wave * (32 * SLD + 32);
+  int* slab_dst = reinterpret_cast<int*>(slab + 32 * SLD);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int trow = tok0 + j * 32 + r32;
-    if (j < jmax && trow < tile.rows) {
-      const float w = ldc(&p.row_w[tile.row0 + trow]);
-      float* yrow = p.y + static_cast<size_t>(ldc(&p.perm[tile.row0 + trow])) * H + n0 + wn * 128;
+    if (j < jmax) {
+      const int myrow = tok0 + j * 32 + r32;
+      float w = 0.0f;
+      if (myrow < tile.rows) w = ldc(&p.row_w[tile.row0 + myrow]);
+      if (kq == 0) slab_dst[r32] = myrow < tile.rows ? ldc(&p.perm[tile.row0 + myrow]) : -1;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          stc16(yrow + i * 32 + g4 * 8 + kq * 4,
-                make_uint4(__float_as_uint(acc[i][j][g4 * 4 + 0] * w),
-                           __float_as_uint(acc[i][j][g4 * 4 + 1] * w),
-                           __float_as_uint(acc[i][j][g4 * 4 + 2] * w),
-                           __float_as_uint(acc[i][j][g4 * 4 + 3] * w)));
-        }
+        for (int g4 = 0; g4 < 4; ++g4)
+          *reinterpret_cast<float4*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) =
+              make_float4(acc[i][j][g4 * 4 + 0] * w, acc[i][j][g4 * 4 + 1] * w,
+                          acc[i][j][g4 * 4 + 2] * w, acc[i][j][g4 * 4 + 3] * w);
+      lds_wave_sync();
+#pragma unroll
+      for (int it = 0; it < 16; ++it) {
+        const int rr = it * 2 + (lane >> 5), cc = (lane & 31) * 4;
+        const int dst = slab_dst[rr];
+        const float4 v = *reinterpret_cast<const float4*>(slab + rr * SLD + cc);
+        if (dst >= 0)
+          st16(p.y + static_cast<size_t>(dst) * H + n0 + wn * 128 + cc,
+               u32x4{__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z),
+                     __float_as_uint(v.w)});
+      }
+      lds_wave_sync();
     }
   }
 }
@@ -497,23 +557,52 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
 __device__ __noinline__ void tiled_combine_task(const Params& p, int blk) {
   const int H = p.H, K = p.K, T = p.T;
   unsigned short* out = reinterpret_cast<unsigned short*>(p.out);
+  const float* y = p.y;
   for (int tl = 0; tl < CMB_TOK; ++tl) {
     const int t = blk * CMB_TOK + tl;
     if (t >= T) break;
-    for (int c = threadIdx.x * 4; c < H; c += T_THREADS * 4) {
-      float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-      for (int k = 0; k < K; ++k) {
-        if (ldc(&p.topk_idx[static_cast<size_t>(t) * K + k]) < 0) continue;
-        const uint4 v = ldc16(p.y + (static_cast<size_t>(t) * K + k) * H + c);
-        s.x += __uint_as_float(v.x);
-        s.y += __uint_as_float(v.y);
-        s.z += __uint_as_float(v.z);
-        s.w += __uint_as_float(v.w);
+    unsigned valid = 0u;  // slots that hold an expert
+    for (int k = 0; k < K; ++k)
+      if (ldc(&p.topk_idx[static_cast<size_t>(t) * K + k]) >= 0) valid |= 1u << k;
+    // two column chunks per pass: 16 row loads of 16 bytes in flight per thread
+    for (int c = threadIdx.x * 4; c < H; c += T_THREADS * 8) {
+      const int c2 = c + T_THREADS * 4;
+      const bool has2 = c2 < H;
+      float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
+      for (int k0 = 0; k0 < K; k0 += 8) {
+        uint4 v[8], u[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (k0 + k < K) {
+            const float* row = y + (static_cast<size_t>(t) * K + k0 + k) * H;
+            v[k] = ld16(row + c);
+            if (has2) u[k] = ld16(row + c2);
+          }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          if (k0 + k < K && ((valid >> (k0 + k)) & 1u)) {
+            s0.x += __uint_as_float(v[k].x);
+            s0.y += __uint_as_float(v[k].y);
+            s0.z += __uint_as_float(v[k].z);
+            s0.w += __uint_as_float(v[k].w);
+            if (has2) {
+              s1.x += __uint_as_float(u[k].x);
+              s1.y += __uint_as_float(u[k].y);
+              s1.z += __uint_as_float(u[k].z);
+              s1.w += __uint_as_float(u[k].w);
+            }
+          }
+        }
       }
-      const unsigned lo = f2bf(s.x) | (f2bf(s.y) << 16);
-      const unsigned hi = f2bf(s.z) | (f2bf(s.w) << 16);
+      unsigned lo = f2bf(s0.x) | (f2bf(s0.y) << 16), hi = f2bf(s0.z) | (f2bf(s0.w) << 16);
       *as_global(reinterpret_cast<unsigned long long*>(out + static_cast<size_t>(t) * H + c)) =
           static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32);
+      if (has2) {
+        lo = f2bf(s1.x) | (f2bf(s1.y) << 16);
+        hi = f2bf(s1.z) | (f2bf(s1.w) << 16);
+        *as_global(reinterpret_cast<unsigned long long*>(out + static_cast<size_t>(t) * H + c2)) =
+            static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32);
+      }
     }
     if ((t & 63) == 0) {
       for (int e = threadIdx.x; e < p.E; e += T_THREADS)
@@ -523,6 +612,21 @@ __device__ __noinline__ void tiled_combine_task(const Params& p, int blk) {
 }
 
 // ---------------------------------------------------------------- worker loop
+// Ticket layout. The prologue (router, scan, scatter) uses one global counter.
+// The GEMM tasks are split into eight queues, one per XCD: queue x owns a
+// contiguous eighth of the row-tile table (which is sorted by expert), first all
+// its gate/up tasks (tile-major), then all its down tasks. A workgroup serves
+// the queue of the XCD it runs on, so tasks that share a token tile or a weight
+// tile run on CUs behind the same L2 at about the same time, and a tile's h
+// rows are consumed where they were produced. A workgroup whose queue is empty
+// steals from the next queue. Dependencies stay inside one queue and point to
+// smaller tickets, so whoever holds them is already running. Combine tasks
+// come from a last global counter once every queue is empty.
+__device__ __forceinline__ int xcc_id() {
+  // HW_REG_XCC_ID (20), bits 0..3
+  return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 7;
+}
+
 __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
   __shared__ WgShared sh;
   if (threadIdx.x == 0) {
@@ -541,97 +645,110 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
   const unsigned nt2 = static_cast<unsigned>(p.H / TN);
   const unsigned ncmb = (T + CMB_TOK - 1u) / CMB_TOK;
   const unsigned n_groups = gridDim.x;
-  unsigned n1 = 0, n2 = 0;
-  bool have_dyn = false, first = true;
+  const int home = xcc_id();
+  bool first = true, ok = true;
 
-  while (true) {
-    const long long t_fetch = p.trace ? wall_clock64() : 0;
-    if (threadIdx.x == 0) sh.ticket = first ? blockIdx.x : n_groups + add_relaxed(&ctl->ticket.v, 1u);
-    first = false;
-    __syncthreads();
-    const unsigned tk = sh.ticket;
-    __syncthreads();
-    unsigned kind = 0, aux = 0;
-    long long t_ready = 0;
-    bool ok = true;
-
-    if (tk < n_rt) {
-      kind = 0;
-      aux = tk;
-      if (p.trace) t_ready = wall_clock64();
-      tiled_router_task(p, static_cast<int>(tk));
-      wg_arrive(&ctl->router_done.v, &sh);
-    } else if (tk == t_scan) {
-      kind = 1;
-      ok = wg_wait_ge(p, &ctl->router_done.v, n_rt, &sh);
-      if (ok) {
-        if (p.trace) t_ready = wall_clock64();
-        tiled_scan_task(p);
-      }
-    } else if (tk < t_dyn0) {
-      kind = 2;
-      aux = tk - t_scatter0;
-      ok = wg_wait_flag(p, FLAG_SCAN, &sh);
-      if (ok) {
-        if (p.trace) t_ready = wall_clock64();
-        tiled_scatter_task(p, static_cast<int>(aux));
-        if (wg_arrive(&ctl->perm_done.v, &sh) == n_rt - 1u) wg_broadcast_flag(p, FLAG_PERM);
-      }
-    } else {
-      if (!have_dyn) {
-        ok = wg_wait_flag(p, FLAG_SCAN, &sh);
-        if (ok) {
-          const unsigned nm = ldc(&ctl->n_mtiles.v);
-          n1 = nm * nt1;
-          n2 = nm * nt2;
-          have_dyn = true;
-        }
-      }
-      const unsigned j = tk - t_dyn0;
-      if (!ok) {
-      } else if (j < n1) {
-        kind = 3;
-        aux = j / nt1;
-        ok = wg_wait_flag(p, FLAG_PERM, &sh);
-        if (ok) {
-          if (p.trace) t_ready = wall_clock64();
-          const TileDesc tile = ld_tile(&p.mtiles[aux]);
-          tiled_gateup_task(p, tile, static_cast<int>(j % nt1));
-          wg_arrive(&p.g1_done[aux].v, &sh);
-        }
-      } else if (j < n1 + n2) {
-        kind = 4;
-        aux = (j - n1) / nt2;
-        ok = wg_wait_ge(p, &p.g1_done[aux].v, nt1, &sh);
-        if (ok) {
-          if (p.trace) t_ready = wall_clock64();
-          const TileDesc tile = ld_tile(&p.mtiles[aux]);
-          tiled_down_task(p, tile, static_cast<int>((j - n1) % nt2));
-          if (wg_arrive(&ctl->g2_done.v, &sh) == n2 - 1u) wg_broadcast_flag(p, FLAG_G2);
-        }
-      } else if (j < n1 + n2 + ncmb) {
-        kind = 5;
-        aux = j - n1 - n2;
-        if (n2 != 0u) ok = wg_wait_flag(p, FLAG_G2, &sh);
-        if (ok) {
-          if (p.trace) t_ready = wall_clock64();
-          tiled_combine_task(p, static_cast<int>(aux));
-        }
-      } else {
-        break;
-      }
-    }
-    if (!ok) break;
-    if (p.trace && threadIdx.x == 0 && tk < p.trace_cap) {
+  auto trace = [&](unsigned id, unsigned kind, unsigned aux, long long t_fetch, long long t_ready) {
+    if (p.trace && threadIdx.x == 0 && id < p.trace_cap) {
       const long long t_end = wall_clock64();
-      TraceRec* r = p.trace + tk;
-      st16(r, u32x4{tk, kind, blockIdx.x, aux});
+      TraceRec* r = p.trace + id;
+      st16(r, u32x4{id, kind, blockIdx.x, aux});
       st16(reinterpret_cast<char*>(r) + 16,
            u32x4{static_cast<unsigned>(t_fetch), static_cast<unsigned>(t_fetch >> 32),
                  static_cast<unsigned>(t_ready), static_cast<unsigned>(t_ready >> 32)});
       st16(reinterpret_cast<char*>(r) + 32,
            u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), 0u, 0u});
     }
+  };
+
+  // ---- prologue: router, scan, scatter from the global counter
+  while (ok) {
+    const long long t_fetch = p.trace ? wall_clock64() : 0;
+    if (threadIdx.x == 0) sh.ticket = first ? blockIdx.x : n_groups + add_relaxed(&ctl->ticket.v, 1u);
+    first = false;
+    __syncthreads();
+    const unsigned tk = sh.ticket;
+    __syncthreads();
+    if (tk >= t_dyn0) break;
+    long long t_ready = 0;
+    if (tk < n_rt) {
+      if (p.trace) t_ready = wall_clock64();
+      tiled_router_task(p, static_cast<int>(tk));
+      wg_arrive<false>(&ctl->router_done.v, &sh);
+      trace(tk, 0, tk, t_fetch, t_ready);
+    } else if (tk == t_scan) {
+      ok = wg_wait_ge(p, &ctl->router_done.v, n_rt, &sh);
+      if (ok) {
+        if (p.trace) t_ready = wall_clock64();
+        tiled_scan_task(p);
+        trace(tk, 1, 0, t_fetch, t_ready);
+      }
+    } else {
+      ok = wg_wait_flag(p, FLAG_SCAN, &sh);
+      if (ok) {
+        if (p.trace) t_ready = wall_clock64();
+        tiled_scatter_task(p, static_cast<int>(tk - t_scatter0));
+        if (wg_arrive<false>(&ctl->perm_done.v, &sh) == n_rt - 1u) wg_broadcast_flag(p, FLAG_PERM);
+        trace(tk, 2, tk - t_scatter0, t_fetch, t_ready);
+      }
+    }
+  }
+
+  // ---- GEMM tasks from the per-XCD queues
+  unsigned nm = 0, n2_total = 0;
+  if (ok) ok = wg_wait_flag(p, FLAG_SCAN, &sh);
+  if (ok) {
+    nm = ldc(&ctl->n_mtiles.v);
+    n2_total = nm * nt2;
+    ok = wg_wait_flag(p, FLAG_PERM, &sh);
+  }
+  for (int hop = 0; ok && hop < 8; ++hop) {
+    const unsigned q = static_cast<unsigned>((home + hop) & 7);
+    const unsigned lo = nm * q / 8u, hi = nm * (q + 1u) / 8u;
+    const unsigned tiles = hi - lo;
+    const unsigned q1 = tiles * nt1, q2 = tiles * nt2;
+    while (ok) {
+      const long long t_fetch = p.trace ? wall_clock64() : 0;
+      if (threadIdx.x == 0) sh.ticket = add_relaxed(&ctl->xq[q].v, 1u);
+      __syncthreads();
+      const unsigned j = sh.ticket;
+      __syncthreads();
+      if (j >= q1 + q2) break;
+      long long t_ready = 0;
+      if (j < q1) {
+        const unsigned m = lo + j / nt1;
+        if (p.trace) t_ready = wall_clock64();
+        const TileDesc tile = ld_tile(&p.mtiles[m]);
+        tiled_gateup_task(p, tile, static_cast<int>(j % nt1));
+        wg_arrive<true>(&p.g1_done[m].v, &sh);
+        trace(t_dyn0 + lo * nt1 + j, 3, m, t_fetch, t_ready);
+      } else {
+        const unsigned jj = j - q1;
+        const unsigned m = lo + jj / nt2;
+        ok = wg_wait_ge(p, &p.g1_done[m].v, nt1, &sh);
+        if (ok) {
+          if (p.trace) t_ready = wall_clock64();
+          const TileDesc tile = ld_tile(&p.mtiles[m]);
+          tiled_down_task(p, tile, static_cast<int>(jj % nt2));
+          if (wg_arrive<true>(&ctl->g2_done.v, &sh) == n2_total - 1u) wg_broadcast_flag(p, FLAG_G2);
+          trace(t_dyn0 + nm * nt1 + lo * nt2 + jj, 4, m, t_fetch, t_ready);
+        }
+      }
+    }
+  }
+
+  // ---- combine tasks from the last global counter
+  if (ok && n2_total != 0u) ok = wg_wait_flag(p, FLAG_G2, &sh);
+  while (ok) {
+    const long long t_fetch = p.trace ? wall_clock64() : 0;
+    if (threadIdx.x == 0) sh.ticket = add_relaxed(&ctl->cticket.v, 1u);
+    __syncthreads();
+    const unsigned c = sh.ticket;
+    __syncthreads();
+    if (c >= ncmb) break;
+    const long long t_ready = p.trace ? wall_clock64() : 0;
+    tiled_combine_task(p, static_cast<int>(c));
+    trace(t_dyn0 + nm * (nt1 + nt2) + c, 5, c, t_fetch, t_ready);
   }
 
   // The last workgroup out returns every counter to zero for the next launch.
@@ -639,13 +756,14 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
   if (threadIdx.x == 0) sh.ok = (add_relaxed(&ctl->exit_count.v, 1u) == n_groups - 1u) ? 1u : 0u;
   __syncthreads();
   if (sh.ok) {
-    const unsigned nm = min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
-    for (unsigned i = threadIdx.x; i < nm; i += T_THREADS) stc(&p.g1_done[i].v, 0u);
+    const unsigned nmr = min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
+    for (unsigned i = threadIdx.x; i < nmr; i += T_THREADS) stc(&p.g1_done[i].v, 0u);
     for (unsigned g = threadIdx.x; g < n_groups; g += T_THREADS) {
       stc(&p.wgflags[g].f[FLAG_SCAN], 0u);
       stc(&p.wgflags[g].f[FLAG_PERM], 0u);
       stc(&p.wgflags[g].f[FLAG_G2], 0u);
     }
+    if (threadIdx.x < 8) stc(&ctl->xq[threadIdx.x].v, 0u);
     if (threadIdx.x == 0) {
       stc(&ctl->launches.v, ldc(&ctl->launches.v) + 1u);
       stc(&ctl->router_done.v, 0u);
@@ -653,6 +771,7 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
       stc(&ctl->g2_done.v, 0u);
       stc(&ctl->n_mtiles.v, 0u);
       stc(&ctl->exit_count.v, 0u);
+      stc(&ctl->cticket.v, 0u);
       stc(&ctl->ticket.v, 0u);
     }
   }
