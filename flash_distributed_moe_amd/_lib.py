@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libflashMoe.so")
 
 F32, BF16 = 0, 1
 SCHED_AUTO, SCHED_STREAM, SCHED_TILED = 0, 1, 2
+FLAG_PACK_WEIGHTS = 1
 HIP_SUCCESS = 0
 HIP_ERROR_INVALID_VALUE = 1
 HIP_ERROR_UNKNOWN = 999
@@ -26,7 +27,7 @@ class LayerDesc(ctypes.Structure):
         ("dtype", ctypes.c_int),
         ("max_tokens", ctypes.c_int),
         ("sched", ctypes.c_int),
-        ("reserved", ctypes.c_int),
+        ("flags", ctypes.c_int),
         ("gate_weights", ctypes.c_void_p),
         ("ffn1_weights", ctypes.c_void_p),
         ("ffn2_weights", ctypes.c_void_p),
@@ -41,6 +42,7 @@ C_ABI = {
                                               ctypes.POINTER(ctypes.c_size_t)]),
     "flashMoeCreate": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(LayerDesc),
                                       ctypes.c_void_p]),
+    "flashMoeRefreshWeights": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p]),
     "flashMoeLaunch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                       ctypes.c_int, ctypes.c_void_p]),
     "flashMoeDestroy": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p]),
@@ -51,6 +53,7 @@ C_ABI = {
                                       ctypes.POINTER(ctypes.c_uint), ctypes.c_void_p]),
     "flashMoeSetWaitLimitMs": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_double]),
     "flashMoeSchedFor": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "flashMoeSetDenseSmallBatch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "flashMoeTraceEnable": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "flashMoeTraceRead": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint,
                                          ctypes.c_void_p]),

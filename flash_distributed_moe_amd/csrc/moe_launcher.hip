@@ -22,6 +22,8 @@
 namespace fmoe {
 hipError_t launch_stream_kernel(const Params& p, int dtype, int grid, hipStream_t stream);
 hipError_t prepare_stream_kernel();
+hipError_t pack_weights(const void* src, void* dst, int dtype, int E, int H, int I, int which,
+                        hipStream_t stream);
 hipError_t launch_tiled_kernel(const Params& p, int grid, hipStream_t stream);
 hipError_t prepare_tiled_kernel();
 int tiled_max_tokens();
@@ -57,7 +59,7 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct Layout {
   size_t ctl, wgflags, g1_done, tok_arrive, cand, topk_idx, topk_w, masks, word_prefix,
-      expert_count, expert_offset, perm, row_w, mtiles, h, y, total;
+      expert_count, expert_offset, perm, row_w, mtiles, h, y, pack1, pack2, total;
   size_t zero_bytes;  // leading region that must be zero before a launch
   int W, max_mtiles;
 };
@@ -92,8 +94,14 @@ Layout make_layout(const FlashMoeLayerDesc& d) {
   L.perm = take(sizeof(int) * rows);
   L.row_w = take(sizeof(float) * rows);
   L.mtiles = take(sizeof(fmoe::TileDesc) * L.max_mtiles);
-  L.h = take(esz * rows * d.intermediate);
+  // h: [rows, I] routed, or [E, 64, I] when small batches run gate/up densely
+  const size_t h_rows = rows > static_cast<size_t>(d.experts) * 64 ? rows
+                                                                    : static_cast<size_t>(d.experts) * 64;
+  L.h = take(esz * h_rows * d.intermediate);
   L.y = take(sizeof(float) * rows * d.hidden);
+  const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
+  L.pack1 = take(pack ? esz * d.experts * 2 * d.intermediate * d.hidden : 0);
+  L.pack2 = take(pack ? esz * d.experts * d.hidden * d.intermediate : 0);
   L.total = off;
   return L;
 }
@@ -123,6 +131,8 @@ hipError_t validate(const FlashMoeLayerDesc* d) {
               d->max_tokens, kMaxRows / d->top_k);
   if (d->sched < FLASH_MOE_SCHED_AUTO || d->sched > FLASH_MOE_SCHED_TILED)
     FMOE_FAIL(hipErrorInvalidValue, "sched = %i", d->sched);
+  if ((d->flags & ~FLASH_MOE_FLAG_PACK_WEIGHTS) != 0)
+    FMOE_FAIL(hipErrorInvalidValue, "unknown flag bits 0x%x", d->flags);
   return hipSuccess;
 }
 
@@ -137,6 +147,7 @@ struct FlashMoeLauncher {
   long long ticks_per_ms = 100000;
   long long spin_limit = 0;
   int last_tokens = 0;
+  bool dense_ok = true;  // small batches may run gate/up for every (expert, token) pair
   fmoe::TraceRec* trace = nullptr;
   unsigned trace_cap = 0;
 };
@@ -156,6 +167,11 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.n_groups = l->num_cus < kMaxGroups ? l->num_cus : kMaxGroups;
   p.n_workers = p.n_groups * 8;
   p.fuse_scatter = (static_cast<long long>(T) * d.top_k <= 2048) ? 1 : 0;
+  // Dense gate/up re-reads every token row for every expert; measured on MI355X
+  // it pays while one 16-row MFMA block holds the whole batch and costs more
+  // than the hidden routing prologue beyond that.
+  p.dense = (T <= 16 && l->dense_ok) ? 1 : 0;
+  p.tpad = (T + 15) / 16 * 16;
   p.max_mtiles = L.max_mtiles;
   p.spin_limit = l->spin_limit;
   p.tokens = tokens;
@@ -163,6 +179,9 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.ffn1 = d.ffn1_weights;
   p.ffn2 = d.ffn2_weights;
   p.bias = d.router_bias;
+  const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
+  p.ffn1_packed = pack ? l->ws + L.pack1 : nullptr;
+  p.ffn2_packed = pack ? l->ws + L.pack2 : nullptr;
   p.out = output;
   char* w = l->ws;
   p.ctl = reinterpret_cast<fmoe::Control*>(w + L.ctl);
@@ -197,6 +216,18 @@ int flashMoeWorkspaceBytes(const FlashMoeLayerDesc* desc, size_t* bytes) {
   if (v != hipSuccess) return v;
   if (bytes == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null result pointer");
   *bytes = make_layout(*desc).total;
+  return hipSuccess;
+}
+
+int flashMoeRefreshWeights(FlashMoeLauncher* l, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (l == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher");
+  const FlashMoeLayerDesc& d = l->desc;
+  if ((d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) == 0) return hipSuccess;  // nothing is copied
+  FMOE_HIP_CHECK(fmoe::pack_weights(d.ffn1_weights, l->ws + l->layout.pack1, d.dtype, d.experts,
+                                    d.hidden, d.intermediate, 0, stream));
+  FMOE_HIP_CHECK(fmoe::pack_weights(d.ffn2_weights, l->ws + l->layout.pack2, d.dtype, d.experts,
+                                    d.hidden, d.intermediate, 1, stream));
   return hipSuccess;
 }
 
@@ -235,6 +266,10 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
   if ((e = hipMalloc(reinterpret_cast<void**>(&l->ws), l->layout.total)) != hipSuccess)
     return fail(e);
   if ((e = hipMemsetAsync(l->ws, 0, l->layout.zero_bytes, stream)) != hipSuccess) return fail(e);
+  if (desc->flags & FLASH_MOE_FLAG_PACK_WEIGHTS) {
+    if ((e = static_cast<hipError_t>(flashMoeRefreshWeights(l, stream))) != hipSuccess)
+      return fail(e);
+  }
   if ((e = hipStreamSynchronize(stream)) != hipSuccess) return fail(e);
   *out = l;
   return hipSuccess;
@@ -354,6 +389,12 @@ int flashMoeTraceRead(FlashMoeLauncher* l, void* records, unsigned max_records, 
   FMOE_HIP_CHECK(hipMemcpy(records, l->trace, sizeof(fmoe::TraceRec) * static_cast<size_t>(n),
                            hipMemcpyDeviceToHost));
   FMOE_HIP_CHECK(hipMemset(l->trace, 0xFF, sizeof(fmoe::TraceRec) * static_cast<size_t>(l->trace_cap)));
+  return hipSuccess;
+}
+
+int flashMoeSetDenseSmallBatch(FlashMoeLauncher* l, int enable) {
+  if (l == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher");
+  l->dense_ok = enable != 0;
   return hipSuccess;
 }
 

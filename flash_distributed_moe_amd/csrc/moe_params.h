@@ -85,6 +85,11 @@ struct Params {
   const void* ffn1;    // [E,2I,H]  rows 0..I-1 gate proj, I..2I-1 up proj
   const void* ffn2;    // [E,H,I]
   const float* bias;   // [E] or null
+  // Optional re-laid-out copies of the expert weights for the streaming variant
+  // (null: read the caller's layout). One gate/up or down wave task reads its
+  // slice front to back: [expert][column block][k-step][weight block][lane][16 B].
+  const void* ffn1_packed;
+  const void* ffn2_packed;
   void* out;           // [T,H], may alias tokens
 
   int* topk_idx;              // [T,K]
@@ -105,6 +110,8 @@ struct Params {
   unsigned* tok_arrive;            // [T] expert groups of the token whose keys are in
   int n_groups;                    // workgroups in the grid
   int fuse_scatter;                // 1: the scan task also writes the permutation
+  int dense;                       // 1: gate/up runs for every (expert, token) pair (small batches)
+  int tpad;                        // dense mode: h rows reserved per expert
   TraceRec* trace;    // null unless tracing; indexed by ticket
   unsigned trace_cap;
 };

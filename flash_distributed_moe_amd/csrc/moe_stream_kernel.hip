@@ -15,7 +15,14 @@
 // Weights stream HBM -> registers -> MFMA with no reuse across waves, which is
 // the right shape when an expert sees at most a few dozen rows (decode).
 // The down projection reads h rows that other workers wrote, so its B operand
-// uses the coherent loads described below.
+// uses coherent loads.
+//
+// Batches of at most 16 tokens run gate/up "dense": every expert is applied to
+// every token (h is [expert][token][I]), which makes the gate/up tasks
+// independent of the router: they start streaming at once and the routing
+// prologue hides behind them. (The code handles up to 64 tokens that way, but
+// beyond one 16-row MFMA block the extra token-row loads cost more bandwidth
+// than the hidden prologue is worth.)
 //
 // Replaces, for this regime, the reference's moeKernel
 // (src/hip/kernel/moeKernel.h:37-107), its task executors
@@ -307,7 +314,9 @@ __device__ void scatter_task(const Params& p, int t) {
 template <typename DT, int NA, int RB, int U, bool COH_B, typename Pre>
 __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[NA],
                                            const typename DT::elem* const (&bp)[RB], int ksteps,
-                                           f32x4 (&acc)[NA][RB], Pre pre) {
+                                           int astep, f32x4 (&acc)[NA][RB], Pre pre) {
+  // astep: elements between one k-step's A fragment and the next (4*EPV in the
+  // caller's row-major layout, NA*64*EPV in the packed layout)
   constexpr int KS = 4 * DT::EPV;
   uint4 a[U][NA], b[U][RB];
 
@@ -315,7 +324,7 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int i = 0; i < NA; ++i) a[u][i] = ld16(ap[i] + static_cast<size_t>(s + u) * KS);
+      for (int i = 0; i < NA; ++i) a[u][i] = ld16(ap[i] + static_cast<size_t>(s + u) * astep);
   };
   auto load_b = [&](int s) {
 #pragma unroll
@@ -358,7 +367,7 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
   for (; s < ksteps; ++s) {  // remainder when ksteps is not a multiple of U
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      const uint4 av = ld16(ap[i] + static_cast<size_t>(s) * KS);
+      const uint4 av = ld16(ap[i] + static_cast<size_t>(s) * astep);
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
         const typename DT::elem* q = bp[r] + static_cast<size_t>(s) * KS;
@@ -373,14 +382,15 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
 // loads of 16 bytes per lane.
 template <int NA, int RB>
 struct RoundSteps {
-  static constexpr int value = RB == 1 ? (NA <= 2 ? 16 : 8) : (RB == 2 ? (NA <= 2 ? 8 : 4) : (NA <= 2 ? 4 : 2));
+  static constexpr int value = RB == 1 ? (NA <= 2 ? 16 : 8) : (RB == 2 ? (NA <= 2 ? 8 : 4) : 4);
 };
 
 // -------------------------------------------------------------------- gate/up
 // h[row, n0 .. n0+16*G1_NB) for the rows of one tile. Follows
 // refExpertFFN1.h:51-65 (two GEMMs against the [2I,H] expert matrix, then
 // SiLU(gate) * up), accumulated on MFMA in float.
-template <typename DT, int RB>
+// DENSE: the tile is (expert, all tokens): row r is token r, h row = row0 + r.
+template <typename DT, int RB, bool DENSE>
 __device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile, int nblk) {
   typedef typename DT::elem elem;
   constexpr int EPV = DT::EPV;
@@ -390,19 +400,30 @@ __device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile, 
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = nblk * (16 * G1_NB);
 
-  const elem* w13 = reinterpret_cast<const elem*>(p.ffn1) +
-                    static_cast<size_t>(tile.expert) * 2 * p.I * p.H;
   const elem* ap[NA];
+  int astep = 4 * EPV;
+  if (p.ffn1_packed != nullptr) {
+    // this task's slice: [k-step][NA blocks][64 lanes][EPV]
+    const size_t task = static_cast<size_t>(tile.expert) * (p.I / (16 * G1_NB)) + nblk;
+    const elem* base = reinterpret_cast<const elem*>(p.ffn1_packed) +
+                       task * (static_cast<size_t>(p.H / (4 * EPV)) * NA * 64 * EPV);
 #pragma unroll
-  for (int b = 0; b < G1_NB; ++b) {
-    ap[b] = w13 + static_cast<size_t>(n0 + 16 * b + r16) * p.H + g * EPV;                // gate
-    ap[G1_NB + b] = w13 + static_cast<size_t>(p.I + n0 + 16 * b + r16) * p.H + g * EPV;  // up
+    for (int i = 0; i < NA; ++i) ap[i] = base + (i * 64 + lane) * EPV;
+    astep = NA * 64 * EPV;
+  } else {
+    const elem* w13 = reinterpret_cast<const elem*>(p.ffn1) +
+                      static_cast<size_t>(tile.expert) * 2 * p.I * p.H;
+#pragma unroll
+    for (int b = 0; b < G1_NB; ++b) {
+      ap[b] = w13 + static_cast<size_t>(n0 + 16 * b + r16) * p.H + g * EPV;                // gate
+      ap[G1_NB + b] = w13 + static_cast<size_t>(p.I + n0 + 16 * b + r16) * p.H + g * EPV;  // up
+    }
   }
   const elem* bp[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
     const int row = min(r * 16 + r16, tile.rows - 1);
-    const int tok = ldc(&p.perm[tile.row0 + row]) / p.K;
+    const int tok = DENSE ? row : ldc(&p.perm[tile.row0 + row]) / p.K;
     bp[r] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(tok) * p.H + g * EPV;
   }
   f32x4 acc[NA][RB];
@@ -411,7 +432,7 @@ __device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile, 
 #pragma unroll
     for (int r = 0; r < RB; ++r) acc[i][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  stream_mma<DT, NA, RB, U, false>(ap, bp, p.H / (4 * EPV), acc, [] { return true; });
+  stream_mma<DT, NA, RB, U, false>(ap, bp, p.H / (4 * EPV), astep, acc, [] { return true; });
 
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
@@ -444,7 +465,7 @@ __device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile, 
 // does (src/hip/kernel/tasks/ffn2Task.h:37-40). The weight rows do not depend
 // on h, so their first loads are issued before the wait for the tile's
 // gate/up tasks. Returns false if that wait failed.
-template <typename DT, int RB>
+template <typename DT, int RB, bool DENSE>
 __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, int nblk, unsigned* dep,
                           unsigned dep_target) {
   typedef typename DT::elem elem;
@@ -455,16 +476,31 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = nblk * (16 * G2_NB);
 
-  const elem* w2 =
-      reinterpret_cast<const elem*>(p.ffn2) + static_cast<size_t>(tile.expert) * p.H * p.I;
   const elem* ap[NA];
+  int astep = 4 * EPV;
+  if (p.ffn2_packed != nullptr) {
+    const size_t task = static_cast<size_t>(tile.expert) * (p.H / (16 * G2_NB)) + nblk;
+    const elem* base = reinterpret_cast<const elem*>(p.ffn2_packed) +
+                       task * (static_cast<size_t>(p.I / (4 * EPV)) * NA * 64 * EPV);
 #pragma unroll
-  for (int b = 0; b < NA; ++b) ap[b] = w2 + static_cast<size_t>(n0 + 16 * b + r16) * p.I + g * EPV;
+    for (int i = 0; i < NA; ++i) ap[i] = base + (i * 64 + lane) * EPV;
+    astep = NA * 64 * EPV;
+  } else {
+    const elem* w2 =
+        reinterpret_cast<const elem*>(p.ffn2) + static_cast<size_t>(tile.expert) * p.H * p.I;
+#pragma unroll
+    for (int b = 0; b < NA; ++b)
+      ap[b] = w2 + static_cast<size_t>(n0 + 16 * b + r16) * p.I + g * EPV;
+  }
   const elem* bp[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
     const int row = min(r * 16 + r16, tile.rows - 1);
-    bp[r] = reinterpret_cast<const elem*>(p.h) + static_cast<size_t>(tile.row0 + row) * p.I + g * EPV;
+    // dense mode: h is [expert][tpad][I] and the row is the token's
+    const size_t hrow = DENSE ? static_cast<size_t>(tile.expert) * p.tpad +
+                                    ldc(&p.perm[tile.row0 + row]) / p.K
+                              : static_cast<size_t>(tile.row0 + row);
+    bp[r] = reinterpret_cast<const elem*>(p.h) + hrow * p.I + g * EPV;
   }
   f32x4 acc[NA][RB];
 #pragma unroll
@@ -472,7 +508,7 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
 #pragma unroll
     for (int r = 0; r < RB; ++r) acc[i][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const bool ok = stream_mma<DT, NA, RB, U, true>(ap, bp, p.I / (4 * EPV), acc, [&] {
+  const bool ok = stream_mma<DT, NA, RB, U, true>(ap, bp, p.I / (4 * EPV), astep, acc, [&] {
     return wave_wait_ge(dep, dep_target, p.ctl, p.spin_limit);
   });
   if (!ok) return false;
@@ -594,8 +630,12 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
   const unsigned n_router = n_dot + T;  // dot tasks, then one select task per token
   const unsigned t_scan = n_router;
   const unsigned t_scatter0 = n_router + 1u;
-  const unsigned t_dyn0 = t_scatter0 + (p.fuse_scatter ? 0u : T);
   const unsigned nt1 = static_cast<unsigned>(p.I / (16 * G1_NB));
+  // dense mode: one gate/up task per (expert, column block), known at launch,
+  // ticketed right after the routing prologue
+  const bool dense = p.dense != 0;
+  const unsigned t_dense0 = t_scatter0 + (p.fuse_scatter ? 0u : T);
+  const unsigned t_dyn0 = t_dense0 + (dense ? static_cast<unsigned>(p.E) * nt1 : 0u);
   const unsigned nt2 = static_cast<unsigned>(p.H / (16 * G2_NB));
   const unsigned ncomb = static_cast<unsigned>((p.H + COMBINE_COLS - 1) / COMBINE_COLS);
   const unsigned worker = blockIdx.x * waves_per_group + wave_in_group;
@@ -635,17 +675,36 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
       if (!wave_wait_ge(&ctl->router_done.v, T, ctl, p.spin_limit)) break;
       if (p.trace) t_ready = wall_clock64();
       scan_task(p);
-    } else if (tk < t_dyn0) {
+    } else if (tk < t_dense0) {
       kind = 2;
       aux = tk - t_scatter0;
       if (!wait_flag(p, FLAG_SCAN, lds_flag, lds_poller)) break;
       if (p.trace) t_ready = wall_clock64();
       scatter_task(p, static_cast<int>(aux));
+    } else if (tk < t_dyn0) {
+      kind = 3;
+      const unsigned j = tk - t_dense0;
+      aux = j / nt1;  // expert
+      if (p.trace) t_ready = wall_clock64();
+      TileDesc tile;
+      tile.expert = static_cast<int>(aux);
+      tile.row0 = static_cast<int>(aux) * p.tpad;
+      tile.rows = p.T;
+      tile.pad = 0;
+      const int nblk = static_cast<int>(j % nt1);
+      if (p.T <= 16) {
+        gateup_task<DT, 1, true>(p, tile, nblk);
+      } else if (p.T <= 32) {
+        gateup_task<DT, 2, true>(p, tile, nblk);
+      } else {
+        gateup_task<DT, 4, true>(p, tile, nblk);
+      }
+      wave_arrive(&p.g1_done[aux].v);
     } else {
       if (!have_dyn) {
         if (!wait_flag(p, FLAG_SCAN, lds_flag, lds_poller)) break;
         const unsigned nm = ldc(&ctl->n_mtiles.v);
-        n1 = nm * nt1;
+        n1 = dense ? 0u : nm * nt1;
         n2 = nm * nt2;
         nc = T * ncomb;
         have_dyn = true;
@@ -662,11 +721,11 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
         const TileDesc tile = ld_tile(&p.mtiles[aux]);
         const int nblk = static_cast<int>(j % nt1);
         if (tile.rows <= 16) {
-          gateup_task<DT, 1>(p, tile, nblk);
+          gateup_task<DT, 1, false>(p, tile, nblk);
         } else if (tile.rows <= 32) {
-          gateup_task<DT, 2>(p, tile, nblk);
+          gateup_task<DT, 2, false>(p, tile, nblk);
         } else {
-          gateup_task<DT, 4>(p, tile, nblk);
+          gateup_task<DT, 4, false>(p, tile, nblk);
         }
         wave_arrive(&p.g1_done[aux].v);
       } else if (j < n1 + n2) {
@@ -675,14 +734,31 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
         const int nblk = static_cast<int>((j - n1) % nt2);
         if (p.trace) t_ready = wall_clock64();
         const TileDesc tile = ld_tile(&p.mtiles[aux]);
-        unsigned* dep = &p.g1_done[aux].v;
         bool ok;
-        if (tile.rows <= 16) {
-          ok = down_task<DT, 1>(p, tile, nblk, dep, nt1);
-        } else if (tile.rows <= 32) {
-          ok = down_task<DT, 2>(p, tile, nblk, dep, nt1);
+        if (dense) {
+          // the expert's gate/up tasks are counted per expert; an expert has one
+          // row tile here (at most 64 rows); the permutation must be final too
+          if (!perm_ready) {
+            if (!wait_flag(p, FLAG_PERM, lds_flag, lds_poller)) break;
+            perm_ready = true;
+          }
+          unsigned* dep = &p.g1_done[tile.expert].v;
+          if (tile.rows <= 16) {
+            ok = down_task<DT, 1, true>(p, tile, nblk, dep, nt1);
+          } else if (tile.rows <= 32) {
+            ok = down_task<DT, 2, true>(p, tile, nblk, dep, nt1);
+          } else {
+            ok = down_task<DT, 4, true>(p, tile, nblk, dep, nt1);
+          }
         } else {
-          ok = down_task<DT, 4>(p, tile, nblk, dep, nt1);
+          unsigned* dep = &p.g1_done[aux].v;
+          if (tile.rows <= 16) {
+            ok = down_task<DT, 1, false>(p, tile, nblk, dep, nt1);
+          } else if (tile.rows <= 32) {
+            ok = down_task<DT, 2, false>(p, tile, nblk, dep, nt1);
+          } else {
+            ok = down_task<DT, 4, false>(p, tile, nblk, dep, nt1);
+          }
         }
         if (!ok) break;
         const unsigned old = wave_arrive(&ctl->g2_done.v);
@@ -722,7 +798,8 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
   }
   last = __builtin_amdgcn_readfirstlane(last);
   if (last) {
-    const unsigned nm = min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
+    unsigned nm = min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
+    if (dense) nm = max(nm, static_cast<unsigned>(p.E));  // counters are per expert there
     for (unsigned i = lane; i < nm; i += 64) stc(&p.g1_done[i].v, 0u);
     for (int g = lane; g < p.n_groups; g += 64) {
       stc(&p.wgflags[g].f[FLAG_SCAN], 0u);
@@ -739,6 +816,55 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
       stc(&ctl->ticket.v, 0u);
     }
   }
+}
+
+// ------------------------------------------------------------ weight packing
+// dst chunk c (16 bytes) of the packed gate/up or down weights <- its source.
+// which = 0: ffn1 [E,2I,H] -> tasks of 2*G1_NB blocks (gate blocks, then up
+// blocks); which = 1: ffn2 [E,H,I] -> tasks of G2_NB blocks.
+template <typename DT>
+__global__ void pack_weights_kernel(const void* src_, void* dst_, int E, int H, int I, int which) {
+  typedef typename DT::elem elem;
+  constexpr int EPV = DT::EPV;
+  const elem* src = reinterpret_cast<const elem*>(src_);
+  const int K = which == 0 ? H : I;            // contraction length
+  const int NA = which == 0 ? 2 * G1_NB : G2_NB;
+  const int nb = which == 0 ? G1_NB : G2_NB;   // 16-row blocks per output slab
+  const int ntask = which == 0 ? I / (16 * G1_NB) : H / (16 * G2_NB);
+  const int ksteps = K / (4 * EPV);
+  const size_t per_task = static_cast<size_t>(ksteps) * NA * 64;
+  const size_t total = static_cast<size_t>(E) * ntask * per_task;
+  for (size_t c = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; c < total;
+       c += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const int lane = static_cast<int>(c & 63);
+    const int a = static_cast<int>((c >> 6) % NA);
+    const int ks = static_cast<int>((c / (64 * NA)) % ksteps);
+    const size_t task = c / per_task;
+    const int nblk = static_cast<int>(task % ntask);
+    const int e = static_cast<int>(task / ntask);
+    const int r16 = lane & 15, g = lane >> 4;
+    size_t row;
+    if (which == 0) {
+      const int n0 = nblk * 16 * nb;
+      row = static_cast<size_t>(e) * 2 * I + (a < nb ? n0 + 16 * a + r16 : I + n0 + 16 * (a - nb) + r16);
+    } else {
+      row = static_cast<size_t>(e) * H + nblk * 16 * nb + 16 * a + r16;
+    }
+    const uint4 v = ld16(src + row * K + static_cast<size_t>(ks) * 4 * EPV + g * EPV);
+    st16(reinterpret_cast<char*>(dst_) + c * 16, u32x4{v.x, v.y, v.z, v.w});
+  }
+}
+
+hipError_t pack_weights(const void* src, void* dst, int dtype, int E, int H, int I, int which,
+                        hipStream_t stream) {
+  if (dtype == DT_BF16) {
+    hipLaunchKernelGGL(pack_weights_kernel<BF16>, dim3(4096), dim3(256), 0, stream, src, dst, E, H, I,
+                       which);
+  } else {
+    hipLaunchKernelGGL(pack_weights_kernel<F32>, dim3(4096), dim3(256), 0, stream, src, dst, E, H, I,
+                       which);
+  }
+  return hipGetLastError();
 }
 
 template __global__ void moe_stream_kernel<F32>(const Params);

@@ -7,7 +7,8 @@ Same argument meaning, checks and error behaviour as the reference binding
 :100-101, "Launcher was destroyed" :45, current torch stream :58,65,93), with
 these additions: bfloat16 tensors are accepted next to float32, and ``create``
 takes optional ``top_k`` (default 8, the reference's compile-time value),
-``router_bias`` and ``sched``. torch supplies device memory and the current
+``router_bias``, ``sched`` and ``pack_weights`` (keep a streaming-friendly second
+copy of the expert weights for small batches). torch supplies device memory and the current
 stream; the work happens behind the C ABI of libflashMoe.so.
 """
 import ctypes
@@ -59,7 +60,8 @@ class MoeKernelLauncher:
         return self._h is not None
 
     def create(self, gate_weights, ffn1_expert_weights, ffn2_expert_weights, max_tokens, uid,
-               rank, world_size, top_k=8, router_bias=None, sched=_lib.SCHED_AUTO):
+               rank, world_size, top_k=8, router_bias=None, sched=_lib.SCHED_AUTO,
+               pack_weights=False):
         _check(self._h is None, "Launcher already created")
         for t, n in ((gate_weights, "gate_weights"), (ffn1_expert_weights, "ffn1_expert_weights"),
                      (ffn2_expert_weights, "ffn2_expert_weights")):
@@ -91,6 +93,7 @@ class MoeKernelLauncher:
         d.experts, d.hidden, d.intermediate, d.top_k = experts, hidden, inter, int(top_k)
         d.dtype = _lib.BF16 if gate_weights.dtype == torch.bfloat16 else _lib.F32
         d.max_tokens, d.sched = int(max_tokens), int(sched)
+        d.flags = _lib.FLAG_PACK_WEIGHTS if pack_weights else 0
         d.gate_weights = gate_weights.data_ptr()
         d.ffn1_weights = ffn1_expert_weights.data_ptr()
         d.ffn2_weights = ffn2_expert_weights.data_ptr()
@@ -169,6 +172,16 @@ class MoeKernelLauncher:
             _hip_check(self._lib.flashMoeTraceRead(self._h, rec.ctypes.data, self._trace_cap,
                                                    _stream()), "flashMoeTraceRead")
         return rec[rec["kind"] != 0xFFFFFFFF]
+
+    def refresh_weights(self):
+        """Re-pack the expert weights after the caller changed them in place."""
+        with torch.cuda.device(self._device):
+            _hip_check(self._lib.flashMoeRefreshWeights(self._h, _stream()),
+                       "flashMoeRefreshWeights")
+
+    def set_dense_small_batch(self, enable):
+        _hip_check(self._lib.flashMoeSetDenseSmallBatch(self._h, 1 if enable else 0),
+                   "flashMoeSetDenseSmallBatch")
 
     def sched_for(self, tokens_num):
         return self._lib.flashMoeSchedFor(self._h, int(tokens_num))

@@ -42,6 +42,13 @@ enum { FLASH_MOE_F32 = 0, FLASH_MOE_BF16 = 1 };
 /* Scheduling variant. AUTO picks by rows per expert. */
 enum { FLASH_MOE_SCHED_AUTO = 0, FLASH_MOE_SCHED_STREAM = 1, FLASH_MOE_SCHED_TILED = 2 };
 
+/* FLASH_MOE_FLAG_PACK_WEIGHTS: at create the expert weights are copied once into
+ * a layout that the streaming (small-batch) variant reads front to back, which
+ * is what HBM likes best; costs a second copy of the expert weights in device
+ * memory. The caller's tensors stay the external format and are still what the
+ * tiled variant reads; after changing them call flashMoeRefreshWeights. */
+enum { FLASH_MOE_FLAG_PACK_WEIGHTS = 1 };
+
 typedef struct FlashMoeLayerDesc {
   int experts;      /* E, 1..256 */
   int hidden;       /* H, multiple of 64 */
@@ -50,7 +57,7 @@ typedef struct FlashMoeLayerDesc {
   int dtype;        /* FLASH_MOE_F32 or FLASH_MOE_BF16: weights, tokens, output */
   int max_tokens;   /* largest tokens_num a launch may pass */
   int sched;        /* FLASH_MOE_SCHED_* */
-  int reserved;
+  int flags;        /* FLASH_MOE_FLAG_* bits */
   const void* gate_weights;  /* device, [E,H] row-major */
   const void* ffn1_weights;  /* device, [E,2I,H]: rows 0..I-1 gate proj, I..2I-1 up proj */
   const void* ffn2_weights;  /* device, [E,H,I] */
@@ -65,6 +72,12 @@ int flashMoeWorkspaceBytes(const FlashMoeLayerDesc* desc, size_t* bytes);
  * untouched. hipErrorUnknown: max_tokens beyond capacity;
  * hipErrorInvalidValue: anything else wrong with the description. */
 int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* stream);
+
+/* Re-reads the caller's expert weights into the packed copy (no-op without
+ * FLASH_MOE_FLAG_PACK_WEIGHTS). Enqueued on `stream`. No counterpart in the
+ * reference, which keeps no copy of the weights
+ * (src/hip/launcher/moeKernelLauncher.hip:107-109). */
+int flashMoeRefreshWeights(FlashMoeLauncher* l, void* stream);
 
 /* Enqueues one forward pass on `stream` and returns without waiting.
  * tokens, output: device [tokens_num, H] in the layer dtype; output may alias
@@ -106,6 +119,12 @@ int flashMoeSetWaitLimitMs(FlashMoeLauncher* l, double ms);
  * max_records records to the host and marks all records unused (all bits set). */
 int flashMoeTraceEnable(FlashMoeLauncher* l, unsigned capacity);
 int flashMoeTraceRead(FlashMoeLauncher* l, void* records, unsigned max_records, void* stream);
+
+/* Batches of at most 16 tokens run the gate/up projection for every (expert,
+ * token) pair so that it does not wait for the router (default on). 0 turns
+ * that off: gate/up then runs only for routed rows, after the router. Results
+ * are identical either way. No counterpart in the reference. */
+int flashMoeSetDenseSmallBatch(FlashMoeLauncher* l, int enable);
 
 /* Which scheduling variant a launch of tokens_num tokens would use. */
 int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num);

@@ -15,7 +15,8 @@ TOL = {"bf16": 1e-2, "f32": 2e-5}
 
 
 class GpuCase:
-    def __init__(self, cfg, seed=7907, sched=_lib.SCHED_AUTO, max_tokens=None, inputs=None):
+    def __init__(self, cfg, seed=7907, sched=_lib.SCHED_AUTO, max_tokens=None, inputs=None,
+                 pack_weights=False):
         self.cfg, self.seed = cfg, seed
         self.dev = torch.device("cuda:0")
         self.inp = inputs or synth.make_inputs_torch(cfg, seed, self.dev)
@@ -23,7 +24,8 @@ class GpuCase:
         uid = self.launcher.getDistributedUniqueId(empty=True)
         self.launcher.create(self.inp["gate"], self.inp["ffn1"], self.inp["ffn2"],
                              max_tokens or cfg.T, uid, 0, 1, top_k=cfg.k,
-                             router_bias=self.inp["bias"], sched=sched)
+                             router_bias=self.inp["bias"], sched=sched,
+                             pack_weights=pack_weights)
 
     def run(self, tokens=None, inplace=False):
         x = self.inp["tokens"] if tokens is None else tokens

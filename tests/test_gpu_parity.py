@@ -133,3 +133,49 @@ def test_tiled_variant_forced(shape):
             other.close()
     finally:
         case.close()
+
+
+@pytest.mark.parametrize("T", [1, 5, 16])
+def test_dense_small_batch_equals_routed(T):
+    """Batches of <= 16 tokens run gate/up for every (expert, token) pair; with
+    that turned off the routed path must give the same bits."""
+    cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=T, name="dense")
+    case = GpuCase(cfg, seed=40 + T)
+    try:
+        x = case.inp["tokens"]
+        dense = case.run()
+        case.check_routing(x, case.launcher.routing(T))
+        case.check_outputs(x, dense)
+        case.launcher.set_dense_small_batch(False)
+        routed = case.run()
+        assert torch.equal(dense, routed)
+        case.launcher.set_dense_small_batch(True)
+        assert torch.equal(case.run(), dense)
+    finally:
+        case.close()
+
+
+@pytest.mark.parametrize("name,T", [("qwen3_30b_decode", 64), ("qwen3_30b_decode", 100),
+                                    ("tiny_f32", 16)])
+def test_packed_weights_equal_unpacked(name, T):
+    """The packed second copy of the expert weights changes where bytes are read
+    from, not what is computed."""
+    cfg = synth.CONFIGS[name].replace(T=T)
+    a = GpuCase(cfg, seed=11)
+    try:
+        b = GpuCase(cfg, seed=11, inputs=a.inp, pack_weights=True)
+        try:
+            out_a, out_b = a.run(), b.run()
+            assert torch.equal(out_a, out_b)
+            b.check_routing(b.inp["tokens"], b.launcher.routing(T))
+            b.check_outputs(b.inp["tokens"], out_b, None if T <= 64 else np.arange(0, T, 7))
+            # refresh after an in-place weight change
+            b.inp["ffn2"].mul_(2.0)
+            b.launcher.refresh_weights()
+            a_out2, b_out2 = a.run(), b.run()
+            assert torch.equal(a_out2, b_out2)
+            b.inp["ffn2"].mul_(0.5)
+        finally:
+            b.close()
+    finally:
+        a.close()
