@@ -86,6 +86,8 @@ def main():
     ap.add_argument("--seed", type=int, default=7907)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sched", type=int, default=0)
+    ap.add_argument("--no-pack-weights", action="store_true",
+                    help="read the caller's weight layout instead of the packed second copy")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs the MoE layer on ONE GPU (no collectives, no "
@@ -108,7 +110,8 @@ def main():
     launcher = MoeKernelLauncher()
     launcher.create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T,
                     launcher.getDistributedUniqueId(empty=True), 0, 1, top_k=cfg.k,
-                    router_bias=inp["bias"], sched=args.sched)
+                    router_bias=inp["bias"], sched=args.sched,
+                    pack_weights=not args.no_pack_weights)
 
     for _ in range(args.warmup):
         launcher.launch(x, out)
@@ -183,7 +186,7 @@ def main():
         "data": "synthetic (seeded Irwin-Hall normal weights sigma 0.02, activations sigma 1)",
         "config": {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E,
                    "top_k": cfg.k, "intermediate": cfg.I, "hot_experts": cfg.hot,
-                   "seed": args.seed},
+                   "seed": args.seed, "packed_weight_copy": not args.no_pack_weights},
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
