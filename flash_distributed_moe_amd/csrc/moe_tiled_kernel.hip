@@ -23,6 +23,8 @@
 // Replaces, for this regime, the reference's moeKernel
 // (src/hip/kernel/moeKernel.h:37-107) and its TILE_M=1 GEMV tiles
 // (src/hip/kernel/tasks/internal/gemmImpl/basicGemmTileImpl.h:14-94).
+#include <type_traits>
+
 #include "moe_device.h"
 
 namespace fmoe {
@@ -31,8 +33,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int TM = 256;            // token rows per tile
 constexpr int TN = 256;            // weight rows per tile
-constexpr int TK = 64;             // k per LDS stage
-constexpr int TLD = TK + 8;        // LDS row stride, bf16 elements (144 bytes)
+constexpr int TK = 32;             // k per LDS stage (one 64-byte row slice)
+constexpr int STAGES = 4;          // LDS stages in flight
+constexpr int STAGE_BYTES = (TM + TN) * TK * 2;  // 32 KiB: weight rows, then token rows
 constexpr int T_THREADS = 256;
 constexpr int G1_COLS = TN / 2;    // h columns per gate/up task
 constexpr int RT_TOK = 32;         // tokens per router / scatter task
@@ -41,7 +44,7 @@ constexpr int RT_XLD = RT_TOK + 4;     // floats per k-row of the transposed tok
 constexpr int RT_WLD = 128 + 4;        // floats per k-row of the transposed expert chunk
 constexpr int CMB_TOK = 8;         // tokens per combine task
 
-constexpr int TILE_LDS_BYTES = 2 * (TM + TN) * TLD * 2;  // 147456
+constexpr int TILE_LDS_BYTES = STAGES * STAGE_BYTES;  // 131072
 constexpr int ROUTER_LDS_BYTES = RT_KC * (RT_XLD + RT_WLD) * 4 + RT_TOK * MAX_EXPERTS * 8 +
                                  4 * SELECT_LDS_BYTES;
 constexpr int TILED_LDS_BYTES = TILE_LDS_BYTES > ROUTER_LDS_BYTES ? TILE_LDS_BYTES : ROUTER_LDS_BYTES;
@@ -307,136 +310,234 @@ __device__ void tiled_scatter_task(const Params& p, int blk) {
 }
 
 // -------------------------------------------------------------- the GEMM tile
-// Per-thread staging map. Each k-step a thread moves 8 chunks of 16 bytes of
-// each operand: chunk q covers stage row (tid/8 + 32*q), bytes (tid%8)*16 of
-// the row's 128-byte k-slice. Weight rows are regular (two bases: stage rows
-// 0..127 and 128..255); token rows are given per chunk (gathered rows).
+// Operands go HBM/L2 -> LDS directly (global_load_lds_dwordx4: lane l's 16
+// bytes land at LDS base + 16*l, from any global address), four stages of 32
+// k deep, so no register staging, no LDS write instructions and almost no VALU
+// work in the loop: with one wave per SIMD every VALU or LDS instruction of a
+// wave delays its next MFMA (measured: 8 cycles between VALU instructions of one
+// wave, ~65 cycles between its ds_read_b128 with 4 waves per CU).
+//
+// Values that are the same in every lane but that the compiler cannot prove so
+// (they come through a struct reference): pin them to scalar registers, so
+// loops and branches on them stay scalar.
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename T>
+__device__ __forceinline__ T* uni(T* ptr) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
+  return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
+
+// LDS stage layout: rows of 64 bytes (32 bf16), unpadded, weight rows 0..255
+// then token rows 0..255. Row R keeps its four 16-byte chunks permuted: chunk C
+// sits at position C ^ ((R >> 1) & 3), so the 8 rows a quarter-wave reads
+// together fall in 8 different 16-byte bank groups. One wave-wide load fills
+// 16 rows; lane l loads the chunk that belongs at position l & 3 of row l >> 2.
 struct TileRows {
-  const unsigned short* w_lo;  // stage row tid/8, this thread's k-chunk
-  const unsigned short* w_hi;  // stage row 128 + tid/8
-  size_t w_step;               // elements between stage rows 32 apart
-  const unsigned short* tbase;
-  int trow[8];                 // source row of token-stage row tid/8 + 32*q
-  size_t tstride;              // elements per source row
-  int lds_off;                 // element offset of chunk 0 inside one operand stage
+  const unsigned char* wbase;  // uniform: expert's weight matrix
+  const unsigned char* tbase;  // uniform: tokens, or this tile's h rows
+  unsigned woff[4];            // byte offset of this lane's chunk of weight-stage row wave*64+q*16+(lane>>2)
+  unsigned toff[4];            // same for the token stage
 };
+
+#define FMOE_G1 __attribute__((address_space(1)))
+#define FMOE_L3 __attribute__((address_space(3)))
 
 __device__ __forceinline__ f32x16 mma32(const uint4& a, const uint4& b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                  __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// wait until at most N of this wave's vector-memory operations are outstanding
+// (they complete in order); nothing else is waited for
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// One wave-wide 16-byte-per-lane load from global memory straight into LDS:
+// lane l's 16 bytes from base + off land at LDS byte address lds_addr + 16*l.
+// Written as assembly so that the compiler does not order LDS reads of other
+// stages behind it; completion is tracked by hand with wait_vm.
+__device__ __forceinline__ void load_to_lds(unsigned off, const unsigned char* base, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(off), "s"(base), "s"(lds_addr)
+               : "memory");
+}
+
+struct Frags {
+  uint4 a[4];  // weight blocks
+  uint4 b[4];  // token blocks
+};
+
+// Interleave hint for one half k-step: one LDS read, then two matrix
+// instructions, eight times over.
+__device__ __forceinline__ void interleave_reads_and_mfma() {
+#pragma unroll
+  for (int n = 0; n < 8; ++n) {
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+  }
+}
+
 // acc[i][j] (+)= W-block i (32 weight rows) x token-block j (32 token rows).
 // wblk[i]: first weight row of block i inside the weight stage; tokens of this
-// wave start at tok0. jmax: token blocks of this wave that hold valid rows.
-// COH_T: the token operand was written by other workers during this launch.
-template <bool COH_T>
+// wave start at tok0. JMAX: token blocks of this wave that are computed.
+// Every wave loads its share of each stage whatever its JMAX.
+template <int JMAX>
+__device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, const int (&wblk)[4],
+                                            int tok0, f32x16 (&acc)[4][4]) {
+  const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
+  const int r32 = lane & 31, kq = lane >> 5;
+  const unsigned char* lds = lds_raw;
+  const unsigned lds_addr = uni(static_cast<unsigned>(
+      reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
+
+  auto issue = [&](int ks) {  // this wave's 8 loads of k-step ks into stage ks % STAGES
+#ifdef FMOE_DBG_NO_GLOBAL    // timing experiment: keep re-reading the first k-steps (cache hits)
+    const int src = ks & 3;
+#else
+    const int src = ks;
+#endif
+    const unsigned st = lds_addr + (ks & (STAGES - 1)) * STAGE_BYTES + wave * 4096;
+    const unsigned char* wsrc = rows.wbase + static_cast<size_t>(src) * (TK * 2);
+    const unsigned char* tsrc = rows.tbase + static_cast<size_t>(src) * (TK * 2);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) load_to_lds(rows.woff[q], wsrc, st + q * 1024);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) load_to_lds(rows.toff[q], tsrc, st + TN * TK * 2 + q * 1024);
+  };
+
+  // per-lane read offsets: row r32 of a block, chunk kk*2+kq at its permuted position
+  const int swz = (r32 >> 1) & 3;
+  const int rd0 = r32 * 64 + ((kq ^ swz) << 4);        // kk = 0
+  const int rd1 = r32 * 64 + (((kq ^ swz) ^ 2) << 4);  // kk = 1
+
+  auto read = [&](Frags& f, int ks, int kk) {
+    const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? rd0 : rd1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (JMAX > 0) f.a[i] = *reinterpret_cast<const uint4*>(st + wblk[i] * 64);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (j < JMAX) f.b[j] = *reinterpret_cast<const uint4*>(st + TN * TK * 2 + (tok0 + j * 32) * 64);
+  };
+  auto mfma = [&](const Frags& f) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (j < JMAX) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#ifdef FMOE_DBG_NO_MFMA  // timing experiment: consume the fragments without the matrix core
+          acc[i][j][0] += __uint_as_float(f.a[i].x ^ f.b[j].y);
+#else
+          acc[i][j] = mma32(f.a[i], f.b[j], acc[i][j]);
+#endif
+        }
+      }
+  };
+
+  // k-step ks: fragments of its first half are in f0 on entry. While the first
+  // half multiplies, the second half is read; while the second half multiplies,
+  // the next stage is confirmed, the stage just finished is refilled, and the
+  // next step's first half is read. PENDING: loads of later stages that may
+  // still be in flight when stage ks+1 has to be complete (8 per stage).
+  Frags f0, f1;
+  auto step = [&](int ks, auto pending_tag, auto refill_tag, auto last_tag) {
+    constexpr int PENDING = decltype(pending_tag)::value;
+    constexpr bool REFILL = decltype(refill_tag)::value;
+    constexpr bool LAST = decltype(last_tag)::value;
+    read(f1, ks, 1);
+    mfma(f0);
+    interleave_reads_and_mfma();
+    __builtin_amdgcn_sched_barrier(0);
+    if (!LAST) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // nobody still reads stage ks after the barrier
+      wait_vm<PENDING>();
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (REFILL) {
+        if (ks + STAGES < ksteps) issue(ks + STAGES);
+      }
+      read(f0, ks + 1, 0);
+    }
+    mfma(f1);
+    interleave_reads_and_mfma();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I8 = std::integral_constant<int, 8>;
+  using I16 = std::integral_constant<int, 16>;
+
+#pragma unroll
+  for (int s = 0; s < STAGES; ++s) issue(s);  // ksteps >= STAGES for every admitted shape
+  wait_vm<24>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  read(f0, 0, 0);
+  int ks = 0;
+  for (; ks + 3 < ksteps; ++ks) step(ks, I16{}, std::true_type{}, std::false_type{});
+  step(ks++, I8{}, std::false_type{}, std::false_type{});
+  step(ks++, I0{}, std::false_type{}, std::false_type{});
+  step(ks, I0{}, std::false_type{}, std::true_type{});
+  __syncthreads();  // the stages are free for the epilogue
+}
+
+// jmax is the same for the whole wave: one straight-line loop body per value.
+// Rounding it up is safe: rows past the tile's end are clamped copies whose
+// results the epilogue drops.
 __device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, const int (&wblk)[4],
                                           int tok0, int jmax, f32x16 (&acc)[4][4]) {
-  unsigned short* wst = reinterpret_cast<unsigned short*>(lds_raw);          // [2][TN][TLD]
-  unsigned short* tst = wst + 2 * TN * TLD;                                  // [2][TM][TLD]
-  const int lane = threadIdx.x & 63;
-  const int r32 = lane & 31, kq = lane >> 5;
-
-  // Two register sets: the loads of k-step ks+2 are issued while ks is computed
-  // and are only needed (to be written to LDS) at the end of ks+1, so they have
-  // two full compute phases to arrive.
-  uint4 wr0[8], tr0[8], wr1[8], tr1[8];
-  auto issue = [&](uint4(&wreg)[8], uint4(&treg)[8], int ks) {
-#ifdef FMOE_DBG_NO_GLOBAL  // timing experiment: only the first two k-steps touch memory
-    if (ks >= 2) return;
-#endif
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      wreg[q] = ld16(rows.w_lo + q * rows.w_step + ks * TK);
-      wreg[q + 4] = ld16(rows.w_hi + q * rows.w_step + ks * TK);
-    }
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const unsigned short* src = rows.tbase + static_cast<size_t>(rows.trow[q]) * rows.tstride + ks * TK;
-      treg[q] = COH_T ? ldc16(src) : ld16(src);
-    }
-  };
-  auto stash = [&](const uint4(&wreg)[8], const uint4(&treg)[8], int buf) {
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      *reinterpret_cast<uint4*>(wst + buf * TN * TLD + rows.lds_off + q * 32 * TLD) = wreg[q];
-      *reinterpret_cast<uint4*>(tst + buf * TM * TLD + rows.lds_off + q * 32 * TLD) = treg[q];
-    }
-  };
-  auto compute = [&](int buf) {
-    const unsigned short* wb = wst + buf * TN * TLD;
-    const unsigned short* tb = tst + buf * TM * TLD;
-#pragma unroll
-    for (int kk = 0; kk < TK / 16; ++kk) {
-      uint4 a[4], b[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        a[i] = *reinterpret_cast<const uint4*>(wb + (wblk[i] + r32) * TLD + kk * 16 + kq * 8);
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (j < jmax)
-          b[j] = *reinterpret_cast<const uint4*>(tb + (tok0 + j * 32 + r32) * TLD + kk * 16 + kq * 8);
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (j < jmax) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-#ifdef FMOE_DBG_NO_MFMA  // timing experiment: consume the fragments without the matrix core
-            acc[i][j][0] += __uint_as_float(a[i].x ^ b[j].y);
-#else
-            acc[i][j] = mma32(a[i], b[j], acc[i][j]);
-#endif
-          }
-        }
-    }
-  };
-
-  issue(wr0, tr0, 0);
-  if (ksteps > 1) issue(wr1, tr1, 1);
-  stash(wr0, tr0, 0);
-  __syncthreads();
-  for (int ks = 0; ks < ksteps; ks += 2) {
-    // even step: LDS buffer 0 holds ks, set 1 holds ks+1 (in flight)
-    if (ks + 2 < ksteps) issue(wr0, tr0, ks + 2);
-    compute(0);
-    if (ks + 1 < ksteps) stash(wr1, tr1, 1);
-    __syncthreads();
-    if (ks + 1 >= ksteps) break;
-    // odd step: LDS buffer 1 holds ks+1, set 0 holds ks+2 (in flight)
-    if (ks + 3 < ksteps) issue(wr1, tr1, ks + 3);
-    compute(1);
-    if (ks + 2 < ksteps) stash(wr0, tr0, 0);
-    __syncthreads();
+  if (jmax > 2) {
+    tile_gemm_j<4>(rows, ksteps, wblk, tok0, acc);
+  } else if (jmax > 0) {
+    tile_gemm_j<2>(rows, ksteps, wblk, tok0, acc);
+  } else {
+    tile_gemm_j<0>(rows, ksteps, wblk, tok0, acc);
   }
+}
+
+// The chunk lane `lane` of wave `wave` loads for stage row wave*64 + q*16 + (lane >> 2):
+// position lane & 3 of that row holds chunk (lane & 3) ^ ((row >> 1) & 3).
+__device__ __forceinline__ int stage_row(int q) {
+  return (threadIdx.x >> 6) * 64 + q * 16 + ((threadIdx.x & 63) >> 2);
+}
+__device__ __forceinline__ unsigned stage_chunk_bytes(int row) {
+  return static_cast<unsigned>(((threadIdx.x & 3) ^ ((row >> 1) & 3)) << 4);
 }
 
 // gate/up: h[row, n0 .. n0+128) for one row tile
 // (test/singleGPU/cpp/moe/reference/refExpertFFN1.h:51-65).
-__device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& tile, int nblk) {
-  const int H = p.H, I = p.I, K = p.K;
-  const int n0 = nblk * G1_COLS;
-  const unsigned short* w13 =
-      reinterpret_cast<const unsigned short*>(p.ffn1) + static_cast<size_t>(tile.expert) * 2 * I * H;
-  const int srow = threadIdx.x >> 3, kc = threadIdx.x & 7;
+__device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& tile_in, int nblk) {
+  const int H = uni(p.H), I = uni(p.I), K = uni(p.K);
+  TileDesc tile;
+  tile.expert = uni(tile_in.expert);
+  tile.row0 = uni(tile_in.row0);
+  tile.rows = uni(tile_in.rows);
+  const int n0 = uni(nblk) * G1_COLS;
+  const unsigned short* w13 = uni(reinterpret_cast<const unsigned short*>(p.ffn1)) +
+                              static_cast<size_t>(tile.expert) * 2 * I * H;
   TileRows rows;
-  // weight stage rows 0..127: gate rows n0+row, 128..255: up rows I+n0+(row-128)
-  rows.w_lo = w13 + static_cast<size_t>(n0 + srow) * H + kc * 8;
-  rows.w_hi = w13 + static_cast<size_t>(I + n0 + srow) * H + kc * 8;
-  rows.w_step = static_cast<size_t>(32) * H;
-  rows.tbase = reinterpret_cast<const unsigned short*>(p.tokens) + kc * 8;
-  rows.tstride = static_cast<size_t>(H);
-  rows.lds_off = srow * TLD + kc * 8;
+  rows.wbase = reinterpret_cast<const unsigned char*>(w13);
+  rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
 #pragma unroll
-  for (int q = 0; q < 8; ++q) {
-    const int tr = min(srow + 32 * q, tile.rows - 1);
-    rows.trow[q] = ldc(&p.perm[tile.row0 + tr]) / K;
+  for (int q = 0; q < 4; ++q) {
+    const int row = stage_row(q);
+    // weight stage rows 0..127: gate rows n0+row, 128..255: up rows I+n0+(row-128)
+    const int wrow = row < G1_COLS ? n0 + row : I + n0 + (row - G1_COLS);
+    rows.woff[q] = static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+    const int tok = ldc(&p.perm[tile.row0 + min(row, tile.rows - 1)]) / K;
+    rows.toff[q] = static_cast<unsigned>(tok) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
   }
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int wn = wave & 1, wm = wave >> 1;
   const int wblk[4] = {wn * 64, wn * 64 + 32, G1_COLS + wn * 64, G1_COLS + wn * 64 + 32};
   const int tok0 = wm * 128;
-  const int jmax = min(4, max(0, (tile.rows - tok0 + 31) / 32));
+  const int jmax = uni(min(4, max(0, (tile.rows - tok0 + 31) / 32)));
+  unsigned short* h = uni(reinterpret_cast<unsigned short*>(p.h)) +
+                      static_cast<size_t>(tile.row0) * I + n0 + wn * 64;
   f32x16 acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -445,12 +546,12 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  tile_gemm<false>(rows, H / TK, wblk, tok0, jmax, acc);
+  tile_gemm(rows, H / TK, wblk, tok0, jmax, acc);
 
   // Epilogue through LDS (the stage buffers are free now): each wave turns its
-  // 32-token x 64-column blocks into full 128-byte row segments of h.
+  // 32-token x 64-column blocks into full 128-byte row segments of h. Nothing
+  // here waits for a store.
   const int r32 = lane & 31, kq = lane >> 5;
-  unsigned short* h = reinterpret_cast<unsigned short*>(p.h);
   constexpr int SLD = 64 + 8;  // slab row stride, bf16 elements
   unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * 32 * SLD;
 #pragma unroll
@@ -476,8 +577,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
         const int trow = tok0 + j * 32 + rr;
         const uint4 v = *reinterpret_cast<const uint4*>(slab + rr * SLD + cc);
         if (trow < tile.rows)
-          st16(h + static_cast<size_t>(tile.row0 + trow) * I + n0 + wn * 64 + cc,
-               u32x4{v.x, v.y, v.z, v.w});
+          st16(h + static_cast<size_t>(trow) * I + cc, u32x4{v.x, v.y, v.z, v.w});
       }
       lds_wave_sync();
     }
@@ -486,26 +586,47 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
 
 // down: y[t*K+slot, n0 .. n0+256) = w * (h[row] . W2[e]^T)
 // (refFullMoe.h:58-65, src/hip/kernel/tasks/ffn2Task.h:37-40).
-__device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& tile, int nblk) {
-  const int H = p.H, I = p.I;
-  const int n0 = nblk * TN;
-  const unsigned short* w2 =
-      reinterpret_cast<const unsigned short*>(p.ffn2) + static_cast<size_t>(tile.expert) * H * I;
-  const int srow = threadIdx.x >> 3, kc = threadIdx.x & 7;
+__device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& tile_in, int nblk) {
+  const int H = uni(p.H), I = uni(p.I);
+  TileDesc tile;
+  tile.expert = uni(tile_in.expert);
+  tile.row0 = uni(tile_in.row0);
+  tile.rows = uni(tile_in.rows);
+  const int n0 = uni(nblk) * TN;
+  const unsigned short* w2 = uni(reinterpret_cast<const unsigned short*>(p.ffn2)) +
+                             static_cast<size_t>(tile.expert) * H * I;
   TileRows rows;
-  rows.w_lo = w2 + static_cast<size_t>(n0 + srow) * I + kc * 8;
-  rows.w_hi = w2 + static_cast<size_t>(n0 + 128 + srow) * I + kc * 8;
-  rows.w_step = static_cast<size_t>(32) * I;
-  rows.tbase = reinterpret_cast<const unsigned short*>(p.h) + kc * 8;
-  rows.tstride = static_cast<size_t>(I);
-  rows.lds_off = srow * TLD + kc * 8;
+  rows.wbase = reinterpret_cast<const unsigned char*>(w2);
+  rows.tbase = reinterpret_cast<const unsigned char*>(
+      uni(reinterpret_cast<const unsigned short*>(p.h)) + static_cast<size_t>(tile.row0) * I);
 #pragma unroll
-  for (int q = 0; q < 8; ++q) rows.trow[q] = tile.row0 + min(srow + 32 * q, tile.rows - 1);
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int q = 0; q < 4; ++q) {
+    const int row = stage_row(q);
+    rows.woff[q] = static_cast<unsigned>(n0 + row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
+    rows.toff[q] = static_cast<unsigned>(min(row, tile.rows - 1)) * static_cast<unsigned>(I * 2) +
+                   stage_chunk_bytes(row);
+  }
+  const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int wn = wave & 1, wm = wave >> 1;
   const int wblk[4] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
   const int tok0 = wm * 128;
-  const int jmax = min(4, max(0, (tile.rows - tok0 + 31) / 32));
+  const int jmax = uni(min(4, max(0, (tile.rows - tok0 + 31) / 32)));
+  const int r32 = lane & 31, kq = lane >> 5;
+  float* y = uni(p.y) + n0 + wn * 128 + (lane & 31) * 4;
+  // gate weight and destination row (token*K + slot) of this lane's row in each token block
+  float roww[4];
+  int dstrow[4];
+  {
+    const float* row_w = uni(p.row_w) + tile.row0;
+    const int* perm = uni(p.perm) + tile.row0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int myrow = tok0 + j * 32 + r32;
+      const bool valid = myrow < tile.rows;
+      roww[j] = valid ? ldc(&row_w[myrow]) : 0.0f;
+      dstrow[j] = valid ? ldc(&perm[myrow]) : -1;
+    }
+  }
   f32x16 acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -514,21 +635,17 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  tile_gemm<false>(rows, I / TK, wblk, tok0, jmax, acc);
+  tile_gemm(rows, I / TK, wblk, tok0, jmax, acc);
 
   // Epilogue through LDS: 32-token x 128-column blocks become 512-byte row
   // segments of y, scaled by the row's gate weight, at the row's (token, slot).
-  const int r32 = lane & 31, kq = lane >> 5;
+  // Nothing here waits for a store.
   constexpr int SLD = 128 + 4;  // slab row stride, floats
-  float* slab = reinterpret_cast<float*>(lds_raw) + wave * (32 * SLD + 32);
-  int* slab_dst = reinterpret_cast<int*>(slab + 32 * SLD);
+  float* slab = reinterpret_cast<float*>(lds_raw) + wave * (32 * SLD);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     if (j < jmax) {
-      const int myrow = tok0 + j * 32 + r32;
-      float w = 0.0f;
-      if (myrow < tile.rows) w = ldc(&p.row_w[tile.row0 + myrow]);
-      if (kq == 0) slab_dst[r32] = myrow < tile.rows ? ldc(&p.perm[tile.row0 + myrow]) : -1;
+      const float w = roww[j];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -539,11 +656,13 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
       lds_wave_sync();
 #pragma unroll
       for (int it = 0; it < 16; ++it) {
-        const int rr = it * 2 + (lane >> 5), cc = (lane & 31) * 4;
-        const int dst = slab_dst[rr];
-        const float4 v = *reinterpret_cast<const float4*>(slab + rr * SLD + cc);
+        // lanes 0..31 store row 2*it, lanes 32..63 row 2*it+1
+        const int d0 = __builtin_amdgcn_readlane(dstrow[j], it * 2);
+        const int d1 = __builtin_amdgcn_readlane(dstrow[j], it * 2 + 1);
+        const int dst = kq ? d1 : d0;
+        const float4 v = *reinterpret_cast<const float4*>(slab + (it * 2 + kq) * SLD + (lane & 31) * 4);
         if (dst >= 0)
-          st16(p.y + static_cast<size_t>(dst) * H + n0 + wn * 128 + cc,
+          st16(y + static_cast<size_t>(dst) * H,
                u32x4{__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z),
                      __float_as_uint(v.w)});
       }
