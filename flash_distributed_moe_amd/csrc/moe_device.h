@@ -331,6 +331,89 @@ __device__ __forceinline__ void router_select(const Params& p, int t,
   lds_wave_sync();
 }
 
+// Order-preserving image of a logit: greater float <=> greater unsigned. Values
+// the reference's strict '>' against lowest() never admits (NaN, -inf,
+// -FLT_MAX) and experts out of range map to 0, which never wins.
+__device__ __forceinline__ unsigned ordered_bits(float v, bool in_range) {
+  const unsigned u = __float_as_uint(v);
+  return (in_range && v > -FLT_MAX) ? ((u & 0x80000000u) ? ~u : (u | 0x80000000u)) : 0u;
+}
+__device__ __forceinline__ float from_ordered_bits(unsigned u) {
+  return __uint_as_float((u & 0x80000000u) ? (u & 0x7FFFFFFFu) : ~u);
+}
+
+// Maximum over the wave, in a scalar register: four cross-lane steps inside
+// each row of 16 lanes, then the four row results.
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
+  auto step = [](unsigned x, unsigned moved) { return x > moved ? x : moved; };
+  v = step(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, true)));   // lane ^ 1
+  v = step(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, true)));   // lane ^ 2
+  v = step(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x141, 0xF, 0xF, true)));  // mirror in 8
+  v = step(v, static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x140, 0xF, 0xF, true)));  // mirror in 16
+  const unsigned r0 = __builtin_amdgcn_readlane(static_cast<int>(v), 0);
+  const unsigned r1 = __builtin_amdgcn_readlane(static_cast<int>(v), 16);
+  const unsigned r2 = __builtin_amdgcn_readlane(static_cast<int>(v), 32);
+  const unsigned r3 = __builtin_amdgcn_readlane(static_cast<int>(v), 48);
+  const unsigned a = r0 > r1 ? r0 : r1, b = r2 > r3 ? r2 : r3;
+  return a > b ? a : b;
+}
+
+// Same routing as router_select, by K rounds of "take the greatest logit that
+// is left, the lowest expert index among equals" (refTopk.h:36-58 keeps the
+// first of equal values because it compares with a strict '>'). val[j] is
+// ordered_bits of expert lane + 64*j. lex: MAX_TOPK doubles of LDS private to
+// the wave.
+__device__ __forceinline__ void router_select_max(const Params& p, int t,
+                                                  unsigned (&val)[MAX_EXPERTS / 64], double* lex) {
+  constexpr int MAXEPL = MAX_EXPERTS / 64;
+  const int lane = lane_id();
+  const int K = p.K;
+  int my_idx = -1;
+  unsigned my_bits = 0u, top_bits = 0u;
+  for (int s = 0; s < K; ++s) {
+    unsigned m = val[0];
+#pragma unroll
+    for (int j = 1; j < MAXEPL; ++j) m = val[j] > m ? val[j] : m;
+    const unsigned best = wave_max_u32(m);
+    if (s == 0) top_bits = best;
+    if (best == 0u) break;  // fewer admissible experts than K: the remaining slots stay -1
+    int e = -1;
+#pragma unroll
+    for (int j = 0; j < MAXEPL; ++j) {
+      if (e < 0) {
+        const unsigned long long owners = __ballot(val[j] == best);
+        if (owners != 0ull) {
+          const int owner = __ffsll(static_cast<long long>(owners)) - 1;
+          e = owner + 64 * j;
+          if (lane == owner) val[j] = 0u;
+        }
+      }
+    }
+    if (lane == s) {
+      my_idx = e;
+      my_bits = best;
+    }
+  }
+  // softmax over the K winners (descending, so the first is the maximum)
+  const float my_val = my_bits != 0u ? from_ordered_bits(my_bits) : -FLT_MAX;
+  const float v0f = top_bits != 0u ? from_ordered_bits(top_bits) : -FLT_MAX;
+  const double ex = lane < K ? exp(static_cast<double>(my_val) - static_cast<double>(v0f)) : 0.0;
+  if (lane < K) lex[lane] = ex;
+  lds_wave_sync();
+  double sum = 0.0;
+  for (int s = 0; s < K; ++s) sum += lex[s];
+  if (lane < K) {
+    const float w = sum <= 0.0 ? static_cast<float>(1.0 / static_cast<double>(K))
+                               : static_cast<float>(ex / sum);
+    stc(&p.topk_idx[static_cast<size_t>(t) * K + lane], my_idx);
+    stc(&p.topk_w[static_cast<size_t>(t) * K + lane], w);
+    if (my_idx >= 0) {
+      or_relaxed(&p.masks[static_cast<size_t>(my_idx) * p.W + (t >> 6)], 1ull << (t & 63));
+    }
+  }
+  lds_wave_sync();
+}
+
 // ------------------------------------------------------------- scan / scatter
 // The tables the scan and scatter tasks work on, held in registers (Params is
 // reached through a generic reference, which every store would force the

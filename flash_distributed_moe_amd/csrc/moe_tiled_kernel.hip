@@ -39,19 +39,27 @@ constexpr int STAGE_BYTES = (TM + TN) * TK * 2;  // 32 KiB: weight rows, then to
 constexpr int T_THREADS = 256;
 constexpr int G1_COLS = TN / 2;    // h columns per gate/up task
 constexpr int RT_TOK = 32;         // tokens per router / scatter task
-constexpr int RT_KC = 64;          // router k-chunk
-constexpr int RT_XLD = RT_TOK + 4;     // floats per k-row of the transposed token chunk
-constexpr int RT_WLD = 128 + 4;        // floats per k-row of the transposed expert chunk
 constexpr int CMB_TOK = 8;         // tokens per combine task
 
 constexpr int TILE_LDS_BYTES = STAGES * STAGE_BYTES;  // 131072
-constexpr int ROUTER_LDS_BYTES = RT_KC * (RT_XLD + RT_WLD) * 4 + RT_TOK * MAX_EXPERTS * 8 +
-                                 4 * SELECT_LDS_BYTES;
+constexpr int ROUTER_LDS_BYTES = RT_TOK * MAX_EXPERTS * 4 + 4 * MAX_TOPK * 8;
 constexpr int TILED_LDS_BYTES = TILE_LDS_BYTES > ROUTER_LDS_BYTES ? TILE_LDS_BYTES : ROUTER_LDS_BYTES;
 
 extern __shared__ __align__(16) unsigned char lds_raw[];
 
 // ---------------------------------------------------------- workgroup helpers
+// Values that are the same in every lane but that the compiler cannot prove so
+// (they come through a struct reference): pin them to scalar registers, so
+// loops and branches on them stay scalar.
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename T>
+__device__ __forceinline__ T* uni(T* ptr) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
+  return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
+
 struct WgShared {  // small static LDS block
   unsigned ticket;
   unsigned ok;
@@ -124,104 +132,98 @@ __device__ __forceinline__ void wg_broadcast_flag(const Params& p, int which) {
 }
 
 // --------------------------------------------------------------------- router
-// Logits as in test/singleGPU/cpp/moe/reference/refGemm.h:21-24 (one chain per
-// output, k ascending; bf16 products are exact in float so fma == mul+add),
-// then selection as in refTopk.h:36-58 / refMoeGate.h:27-30.
+// Logits as in test/singleGPU/cpp/moe/reference/refGemm.h:21-24: one chain per
+// output, k ascending, one rounding per step. The chain runs on the matrix
+// core: V_MFMA_F32_16X16X1_4B_F32 adds exactly one product per output and
+// instruction, and a product of two bf16 values is exact in float, so every
+// step is the oracle's acc = fmaf(x, w, acc). Each wave carries 16 tokens x 64
+// experts (four 16x16 blocks that share the token operand); every lane streams
+// its own token row and its own expert row from global memory, 32 k at a time.
+// Then selection as in refTopk.h:36-58 / refMoeGate.h:27-30.
 __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
-  const int T = p.T, E = p.E, H = p.H;
-  const unsigned short* tokens = reinterpret_cast<const unsigned short*>(p.tokens);
-  const unsigned short* gate = reinterpret_cast<const unsigned short*>(p.gate);
-  float* xT = reinterpret_cast<float*>(lds_raw);   // [RT_KC][RT_XLD]
-  float* wT = xT + RT_KC * RT_XLD;                 // [RT_KC][RT_WLD]
-  unsigned long long* keys = reinterpret_cast<unsigned long long*>(wT + RT_KC * RT_WLD);
-  unsigned long long* sel = keys + RT_TOK * MAX_EXPERTS;  // 4 waves x SELECT_LDS_BYTES
+  const int T = uni(p.T), E = uni(p.E), H = uni(p.H);
+  const unsigned short* tokens = uni(reinterpret_cast<const unsigned short*>(p.tokens));
+  const unsigned short* gate = uni(reinterpret_cast<const unsigned short*>(p.gate));
+  const float* bias = uni(p.bias);
+  unsigned* keys = reinterpret_cast<unsigned*>(lds_raw);  // [RT_TOK][MAX_EXPERTS] ordered logits
+  double* sel = reinterpret_cast<double*>(keys + RT_TOK * MAX_EXPERTS);  // 4 waves x MAX_TOPK
   const int tid = threadIdx.x;
-  const int tt = tid >> 5, te = tid & 31;          // 4 tokens x 4 experts per thread
-  const int t0 = blk * RT_TOK;
+  const int wave = uni(tid >> 6), lane = tid & 63;
+  const int th = wave >> 1, eh = wave & 1;
+  const int t0 = uni(blk) * RT_TOK;
+  const int l16 = lane & 15, lq = lane >> 4;
+  const unsigned short* xrow =
+      tokens + static_cast<size_t>(min(t0 + th * 16 + l16, T - 1)) * H;
 
   for (int e0 = 0; e0 < E; e0 += 128) {
-    float acc[4][4];
+    const unsigned short* wrow =
+        gate + static_cast<size_t>(min(e0 + eh * 64 + lane, E - 1)) * H;
+    f32x16 acc;
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    uint4 xr[4][4], wr[4][4];  // ring of four 32-k chunks, loads three chunks ahead
+    auto load = [&](int slot, int k) {
+      const int kc = min(k, H - 32);  // past the end: re-read the last chunk
 #pragma unroll
-      for (int b = 0; b < 4; ++b) acc[a][b] = 0.0f;
-
-    // staging map: one token chunk and four expert chunks of 16 bytes per thread
-    const int xr = tid & 31, xc = tid >> 5;
-    const unsigned short* xsrc =
-        tokens + static_cast<size_t>(min(t0 + xr, T - 1)) * H + xc * 8;
-    const unsigned short* wsrc[4];
-    int wr[4], wc[4];
+      for (int c = 0; c < 4; ++c) {
+        xr[slot][c] = ld16(xrow + kc + c * 8);
+        wr[slot][c] = ld16(wrow + kc + c * 8);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the chain they overlap
+    };
+    auto chain = [&](int slot) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int c = tid + 256 * q;
-      wr[q] = c & 127;
-      wc[q] = c >> 7;
-      wsrc[q] = gate + static_cast<size_t>(min(e0 + wr[q], E - 1)) * H + wc[q] * 8;
-    }
-    uint4 xv = ld16(xsrc);
-    uint4 wv[4];
+      for (int c = 0; c < 4; ++c) {
+        const unsigned xw[4] = {xr[slot][c].x, xr[slot][c].y, xr[slot][c].z, xr[slot][c].w};
+        const unsigned ww[4] = {wr[slot][c].x, wr[slot][c].y, wr[slot][c].z, wr[slot][c].w};
 #pragma unroll
-    for (int q = 0; q < 4; ++q) wv[q] = ld16(wsrc[q]);
-
-    for (int k0 = 0; k0 < H; k0 += RT_KC) {
-      __syncthreads();  // previous chunk fully consumed
-      {
-        float f[8];
-        unpack<BF16>(xv, f);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) xT[(xc * 8 + i) * RT_XLD + xr] = f[i];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          unpack<BF16>(wv[q], f);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) wT[(wc[q] * 8 + i) * RT_WLD + wr[q]] = f[i];
+        for (int i = 0; i < 4; ++i) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x1f32(bf16_lo(xw[i]), bf16_lo(ww[i]), acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x1f32(bf16_hi(xw[i]), bf16_hi(ww[i]), acc, 0, 0, 0);
         }
       }
-      __syncthreads();
-      if (k0 + RT_KC < H) {
-        xv = ld16(xsrc + k0 + RT_KC);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    load(0, 0);
+    load(1, 32);
+    load(2, 64);
+    for (int k0 = 0; k0 < H; k0 += 128) {
+      load(3, k0 + 96);
+      chain(0);
+      load(0, k0 + 128);
+      chain(1);
+      load(1, k0 + 160);
+      chain(2);
+      load(2, k0 + 192);
+      chain(3);
+    }
+    // acc[4*b + r] of lane l: token th*16 + 4*(l/16) + r, expert e0 + eh*64 + 16*b + l%16
 #pragma unroll
-        for (int q = 0; q < 4; ++q) wv[q] = ld16(wsrc[q] + k0 + RT_KC);
-      }
-#pragma unroll 8
-      for (int k = 0; k < RT_KC; ++k) {
-        const float4 x4 = *reinterpret_cast<const float4*>(xT + k * RT_XLD + tt * 4);
-        const float4 w4 = *reinterpret_cast<const float4*>(wT + k * RT_WLD + te * 4);
-        const float xa[4] = {x4.x, x4.y, x4.z, x4.w};
-        const float wa[4] = {w4.x, w4.y, w4.z, w4.w};
+    for (int b = 0; b < 4; ++b) {
+      const int e = e0 + eh * 64 + 16 * b + l16;
+      const float bv = (bias != nullptr && e < E) ? as_global(bias)[e] : 0.0f;
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
-#pragma unroll
-          for (int b = 0; b < 4; ++b) acc[a][b] = __builtin_fmaf(xa[a], wa[b], acc[a][b]);
+      for (int r = 0; r < 4; ++r) {
+        float v = acc[4 * b + r];
+        if (bias != nullptr) v = __fadd_rn(v, bv);
+        if (e < MAX_EXPERTS) keys[(th * 16 + 4 * lq + r) * MAX_EXPERTS + e] = ordered_bits(v, e < E);
       }
     }
-    // keys of this expert slab into LDS: keys[token][expert]
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int e = e0 + te * 4 + b;
-        float v = acc[a][b];
-        if (p.bias != nullptr && e < E) v = __fadd_rn(v, as_global(p.bias)[e]);
-        if (e < MAX_EXPERTS) keys[(tt * 4 + a) * MAX_EXPERTS + e] = make_key(v, e, e < E);
-      }
   }
   __syncthreads();
   // selection: each wave takes 8 of the 32 tokens
-  const int wave = tid >> 6, lane = tid & 63;
-  unsigned long long* lk = sel + wave * (SELECT_LDS_BYTES / 8);
+  double* lex = sel + wave * MAX_TOPK;
   for (int i = 0; i < RT_TOK / 4; ++i) {
     const int tl = wave * (RT_TOK / 4) + i;
     const int t = t0 + tl;
     if (t < T) {
-      unsigned long long key[MAX_EXPERTS / 64];
+      unsigned val[MAX_EXPERTS / 64];
 #pragma unroll
       for (int j = 0; j < MAX_EXPERTS / 64; ++j) {
         const int e = lane + 64 * j;
-        key[j] = e < E ? keys[tl * MAX_EXPERTS + e] : 0ull;
+        val[j] = e < E ? keys[tl * MAX_EXPERTS + e] : 0u;
       }
-      router_select(p, t, key, lk);
+      router_select_max(p, t, val, lex);
     }
   }
 }
@@ -317,22 +319,10 @@ __device__ void tiled_scatter_task(const Params& p, int blk) {
 // wave delays its next MFMA (measured: 8 cycles between VALU instructions of one
 // wave, ~65 cycles between its ds_read_b128 with 4 waves per CU).
 //
-// Values that are the same in every lane but that the compiler cannot prove so
-// (they come through a struct reference): pin them to scalar registers, so
-// loops and branches on them stay scalar.
-__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
-template <typename T>
-__device__ __forceinline__ T* uni(T* ptr) {
-  const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
-  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
-  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
-  return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
-}
-
 // LDS stage layout: rows of 64 bytes (32 bf16), unpadded, weight rows 0..255
 // then token rows 0..255. Row R keeps its four 16-byte chunks permuted: chunk C
-// sits at position C ^ ((R >> 1) & 3), so the 8 rows a quarter-wave reads
-// together fall in 8 different 16-byte bank groups. One wave-wide load fills
+// sits at position C ^ ((R >> 2) & 3), so the 16 rows a quarter-wave reads
+// together (256 bytes, all 64 banks) fall in 16 different 16-byte bank groups. One wave-wide load fills
 // 16 rows; lane l loads the chunk that belongs at position l & 3 of row l >> 2.
 struct TileRows {
   const unsigned char* wbase;  // uniform: expert's weight matrix
@@ -367,6 +357,15 @@ __device__ __forceinline__ void load_to_lds(unsigned off, const unsigned char* b
                : "memory");
 }
 
+#ifdef FMOE_DBG_STALL  // timing experiment: cycles a wave spends in the load wait and in the barrier
+__device__ unsigned long long g_stall[4];
+__device__ __forceinline__ unsigned long long stall_clock() {
+  const unsigned long long t = __builtin_amdgcn_s_memtime();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  return t;
+}
+#endif
+
 struct Frags {
   uint4 a[4];  // weight blocks
   uint4 b[4];  // token blocks
@@ -395,77 +394,119 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   const unsigned lds_addr = uni(static_cast<unsigned>(
       reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
 
-  auto issue = [&](int ks) {  // this wave's 8 loads of k-step ks into stage ks % STAGES
-#ifdef FMOE_DBG_NO_GLOBAL    // timing experiment: keep re-reading the first k-steps (cache hits)
+  // load q (0..3: weight rows, 4..7: token rows) of this wave's 8 loads of
+  // k-step ks into stage ks % STAGES
+  auto issue_one = [&](int ks, int q) {
+#ifdef FMOE_DBG_NO_GLOBAL  // timing experiment: keep re-reading the first k-steps (cache hits)
     const int src = ks & 3;
 #else
     const int src = ks;
 #endif
     const unsigned st = lds_addr + (ks & (STAGES - 1)) * STAGE_BYTES + wave * 4096;
-    const unsigned char* wsrc = rows.wbase + static_cast<size_t>(src) * (TK * 2);
-    const unsigned char* tsrc = rows.tbase + static_cast<size_t>(src) * (TK * 2);
+    if (q < 4) {
+      load_to_lds(rows.woff[q], rows.wbase + static_cast<size_t>(src) * (TK * 2), st + q * 1024);
+    } else {
+      load_to_lds(rows.toff[q - 4], rows.tbase + static_cast<size_t>(src) * (TK * 2),
+                  st + TN * TK * 2 + (q - 4) * 1024);
+    }
+  };
+  auto issue = [&](int ks) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) load_to_lds(rows.woff[q], wsrc, st + q * 1024);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) load_to_lds(rows.toff[q], tsrc, st + TN * TK * 2 + q * 1024);
+    for (int q = 0; q < 8; ++q) issue_one(ks, q);
   };
 
   // per-lane read offsets: row r32 of a block, chunk kk*2+kq at its permuted position
-  const int swz = (r32 >> 1) & 3;
+  const int swz = (r32 >> 2) & 3;
   const int rd0 = r32 * 64 + ((kq ^ swz) << 4);        // kk = 0
   const int rd1 = r32 * 64 + (((kq ^ swz) ^ 2) << 4);  // kk = 1
 
-  auto read = [&](Frags& f, int ks, int kk) {
+  auto read_a = [&](Frags& f, int ks, int kk, int i) {
     const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? rd0 : rd1);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (JMAX > 0) f.a[i] = *reinterpret_cast<const uint4*>(st + wblk[i] * 64);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (j < JMAX) f.b[j] = *reinterpret_cast<const uint4*>(st + TN * TK * 2 + (tok0 + j * 32) * 64);
+    if (JMAX > 0) f.a[i] = *reinterpret_cast<const uint4*>(st + wblk[i] * 64);
   };
-  auto mfma = [&](const Frags& f) {
+  auto read_b = [&](Frags& f, int ks, int kk, int j) {
+    const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? rd0 : rd1);
+    if (j < JMAX) f.b[j] = *reinterpret_cast<const uint4*>(st + TN * TK * 2 + (tok0 + j * 32) * 64);
+  };
+  auto read = [&](Frags& f, int ks, int kk) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (j < JMAX) {
+    for (int i = 0; i < 4; ++i) read_a(f, ks, kk, i);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+    for (int j = 0; j < 4; ++j) read_b(f, ks, kk, j);
+  };
+  auto mfma_block = [&](const Frags& f, int j) {
+    if (j < JMAX) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
 #ifdef FMOE_DBG_NO_MFMA  // timing experiment: consume the fragments without the matrix core
-          acc[i][j][0] += __uint_as_float(f.a[i].x ^ f.b[j].y);
+        acc[i][j][0] += __uint_as_float(f.a[i].x ^ f.b[j].y);
 #else
-          acc[i][j] = mma32(f.a[i], f.b[j], acc[i][j]);
+        acc[i][j] = mma32(f.a[i], f.b[j], acc[i][j]);
 #endif
-        }
       }
+    }
   };
 
   // k-step ks: fragments of its first half are in f0 on entry. While the first
   // half multiplies, the second half is read; while the second half multiplies,
   // the next stage is confirmed, the stage just finished is refilled, and the
-  // next step's first half is read. PENDING: loads of later stages that may
-  // still be in flight when stage ks+1 has to be complete (8 per stage).
+  // next step's first half is read — loads and reads spread between the matrix
+  // instructions. PENDING: loads of later stages that may still be in flight
+  // when stage ks+1 has to be complete (8 per stage).
   Frags f0, f1;
+#ifdef FMOE_DBG_STALL
+  unsigned long long stall_vm = 0, stall_bar = 0;
+  const unsigned long long loop_c0 = stall_clock();
+#endif
   auto step = [&](int ks, auto pending_tag, auto refill_tag, auto last_tag) {
     constexpr int PENDING = decltype(pending_tag)::value;
     constexpr bool REFILL = decltype(refill_tag)::value;
     constexpr bool LAST = decltype(last_tag)::value;
+#ifndef FMOE_DBG_NO_READS
     read(f1, ks, 1);
-    mfma(f0);
+#else
+    if (ks == 0) read(f1, ks, 1);
+#endif
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mfma_block(f0, j);
     interleave_reads_and_mfma();
     __builtin_amdgcn_sched_barrier(0);
     if (!LAST) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // nobody still reads stage ks after the barrier
+#ifdef FMOE_DBG_STALL
+      const unsigned long long c0 = stall_clock();
+#endif
       wait_vm<PENDING>();
+#ifdef FMOE_DBG_STALL
+      const unsigned long long c1 = stall_clock();
+#endif
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
-      if (REFILL) {
-        if (ks + STAGES < ksteps) issue(ks + STAGES);
+#ifdef FMOE_DBG_STALL
+      const unsigned long long c2 = stall_clock();
+      stall_vm += c1 - c0;
+      stall_bar += c2 - c1;
+#endif
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        mfma_block(f1, g);
+        __builtin_amdgcn_sched_barrier(0);
+#ifndef FMOE_DBG_NO_REFILL  // timing experiment: the main loop issues no loads
+        if (REFILL) {
+          issue_one(ks + STAGES, 2 * g);
+          issue_one(ks + STAGES, 2 * g + 1);
+        }
+#endif
+#ifndef FMOE_DBG_NO_READS  // timing experiment: the main loop reads no fragments
+        read_a(f0, ks + 1, 0, g);
+        read_b(f0, ks + 1, 0, g);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
       }
-      read(f0, ks + 1, 0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mfma_block(f1, j);
     }
-    mfma(f1);
-    interleave_reads_and_mfma();
-    __builtin_amdgcn_sched_barrier(0);
   };
   using I0 = std::integral_constant<int, 0>;
   using I8 = std::integral_constant<int, 8>;
@@ -478,10 +519,19 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   asm volatile("" ::: "memory");
   read(f0, 0, 0);
   int ks = 0;
-  for (; ks + 3 < ksteps; ++ks) step(ks, I16{}, std::true_type{}, std::false_type{});
+  for (; ks + STAGES < ksteps; ++ks) step(ks, I16{}, std::true_type{}, std::false_type{});
+  step(ks++, I16{}, std::false_type{}, std::false_type{});
   step(ks++, I8{}, std::false_type{}, std::false_type{});
   step(ks++, I0{}, std::false_type{}, std::false_type{});
   step(ks, I0{}, std::false_type{}, std::true_type{});
+#ifdef FMOE_DBG_STALL
+  if (lane == 0) {
+    atomicAdd(&g_stall[0], stall_vm);
+    atomicAdd(&g_stall[1], stall_bar);
+    atomicAdd(&g_stall[2], stall_clock() - loop_c0);
+    atomicAdd(&g_stall[3], 1ull);
+  }
+#endif
   __syncthreads();  // the stages are free for the epilogue
 }
 
@@ -500,12 +550,12 @@ __device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, cons
 }
 
 // The chunk lane `lane` of wave `wave` loads for stage row wave*64 + q*16 + (lane >> 2):
-// position lane & 3 of that row holds chunk (lane & 3) ^ ((row >> 1) & 3).
+// position lane & 3 of that row holds chunk (lane & 3) ^ ((row >> 2) & 3).
 __device__ __forceinline__ int stage_row(int q) {
   return (threadIdx.x >> 6) * 64 + q * 16 + ((threadIdx.x & 63) >> 2);
 }
 __device__ __forceinline__ unsigned stage_chunk_bytes(int row) {
-  return static_cast<unsigned>(((threadIdx.x & 3) ^ ((row >> 1) & 3)) << 4);
+  return static_cast<unsigned>(((threadIdx.x & 3) ^ ((row >> 2) & 3)) << 4);
 }
 
 // gate/up: h[row, n0 .. n0+128) for one row tile
@@ -612,7 +662,8 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
   const int tok0 = wm * 128;
   const int jmax = uni(min(4, max(0, (tile.rows - tok0 + 31) / 32)));
   const int r32 = lane & 31, kq = lane >> 5;
-  float* y = uni(p.y) + n0 + wn * 128 + (lane & 31) * 4;
+  // y rows are bf16 here: H values per (token, slot)
+  unsigned short* y = uni(reinterpret_cast<unsigned short*>(p.y)) + n0 + wn * 128 + (lane & 15) * 8;
   // gate weight and destination row (token*K + slot) of this lane's row in each token block
   float roww[4];
   int dstrow[4];
@@ -637,11 +688,11 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
 
   tile_gemm(rows, I / TK, wblk, tok0, jmax, acc);
 
-  // Epilogue through LDS: 32-token x 128-column blocks become 512-byte row
-  // segments of y, scaled by the row's gate weight, at the row's (token, slot).
-  // Nothing here waits for a store.
-  constexpr int SLD = 128 + 4;  // slab row stride, floats
-  float* slab = reinterpret_cast<float*>(lds_raw) + wave * (32 * SLD);
+  // Epilogue through LDS: 32-token x 128-column blocks become 256-byte row
+  // segments of y (bf16), scaled by the row's gate weight, at the row's
+  // (token, slot). Nothing here waits for a store.
+  constexpr int SLD = 128 + 8;  // slab row stride, bf16 elements
+  unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * (32 * SLD);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     if (j < jmax) {
@@ -649,22 +700,24 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4)
-          *reinterpret_cast<float4*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) =
-              make_float4(acc[i][j][g4 * 4 + 0] * w, acc[i][j][g4 * 4 + 1] * w,
-                          acc[i][j][g4 * 4 + 2] * w, acc[i][j][g4 * 4 + 3] * w);
+        for (int g4 = 0; g4 < 4; ++g4) {
+          uint2 pk;
+          pk.x = f2bf(acc[i][j][g4 * 4 + 0] * w) | (f2bf(acc[i][j][g4 * 4 + 1] * w) << 16);
+          pk.y = f2bf(acc[i][j][g4 * 4 + 2] * w) | (f2bf(acc[i][j][g4 * 4 + 3] * w) << 16);
+          *reinterpret_cast<uint2*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) = pk;
+        }
       lds_wave_sync();
 #pragma unroll
-      for (int it = 0; it < 16; ++it) {
-        // lanes 0..31 store row 2*it, lanes 32..63 row 2*it+1
-        const int d0 = __builtin_amdgcn_readlane(dstrow[j], it * 2);
-        const int d1 = __builtin_amdgcn_readlane(dstrow[j], it * 2 + 1);
-        const int dst = kq ? d1 : d0;
-        const float4 v = *reinterpret_cast<const float4*>(slab + (it * 2 + kq) * SLD + (lane & 31) * 4);
-        if (dst >= 0)
-          st16(y + static_cast<size_t>(dst) * H,
-               u32x4{__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z),
-                     __float_as_uint(v.w)});
+      for (int it = 0; it < 8; ++it) {
+        // each quarter-wave stores one row: rows 4*it .. 4*it+3
+        const int q = lane >> 4;
+        const int d0 = __builtin_amdgcn_readlane(dstrow[j], it * 4);
+        const int d1 = __builtin_amdgcn_readlane(dstrow[j], it * 4 + 1);
+        const int d2 = __builtin_amdgcn_readlane(dstrow[j], it * 4 + 2);
+        const int d3 = __builtin_amdgcn_readlane(dstrow[j], it * 4 + 3);
+        const int dst = q == 0 ? d0 : q == 1 ? d1 : q == 2 ? d2 : d3;
+        const uint4 v = *reinterpret_cast<const uint4*>(slab + (it * 4 + q) * SLD + (lane & 15) * 8);
+        if (dst >= 0) st16(y + static_cast<size_t>(dst) * H, u32x4{v.x, v.y, v.z, v.w});
       }
       lds_wave_sync();
     }
@@ -674,60 +727,52 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
 // combine: out[t] = sum over slots, in slot order, of y[t*K+slot]
 // (refFullMoe.h:35,62-65).
 __device__ __noinline__ void tiled_combine_task(const Params& p, int blk) {
-  const int H = p.H, K = p.K, T = p.T;
-  unsigned short* out = reinterpret_cast<unsigned short*>(p.out);
-  const float* y = p.y;
-  for (int tl = 0; tl < CMB_TOK; ++tl) {
-    const int t = blk * CMB_TOK + tl;
-    if (t >= T) break;
-    unsigned valid = 0u;  // slots that hold an expert
-    for (int k = 0; k < K; ++k)
-      if (ldc(&p.topk_idx[static_cast<size_t>(t) * K + k]) >= 0) valid |= 1u << k;
-    // two column chunks per pass: 16 row loads of 16 bytes in flight per thread
-    for (int c = threadIdx.x * 4; c < H; c += T_THREADS * 8) {
-      const int c2 = c + T_THREADS * 4;
-      const bool has2 = c2 < H;
-      float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
+  const int H = uni(p.H), K = uni(p.K), T = uni(p.T), E = uni(p.E), W = uni(p.W);
+  unsigned short* out = uni(reinterpret_cast<unsigned short*>(p.out));
+  const unsigned short* y = uni(reinterpret_cast<const unsigned short*>(p.y));
+  const int* topk_idx = uni(p.topk_idx);
+  unsigned long long* masks = uni(p.masks);
+  const int tid = threadIdx.x;
+  const int t0 = uni(blk) * CMB_TOK;
+  const int ntok = min(CMB_TOK, T - t0);
+  // which (token, slot) pairs of this task hold an expert: one load each
+  unsigned char* flag = lds_raw;  // [CMB_TOK * MAX_TOPK]
+  if (tid < ntok * K) flag[tid] = ldc(&topk_idx[static_cast<size_t>(t0) * K + tid]) >= 0 ? 1 : 0;
+  __syncthreads();
+  for (int tl = 0; tl < ntok; ++tl) {
+    const int t = t0 + tl;
+    unsigned valid = 0u;
+    for (int k = 0; k < K; ++k) valid |= static_cast<unsigned>(flag[tl * K + k]) << k;
+    valid = uni(static_cast<int>(valid));
+    const unsigned short* yrow = y + static_cast<size_t>(t) * K * H;
+    // 8 columns per thread and pass; the K row loads of a pass are in flight together
+    for (int c = tid * 8; c < H; c += T_THREADS * 8) {
+      float s[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s[i] = 0.0f;
       for (int k0 = 0; k0 < K; k0 += 8) {
-        uint4 v[8], u[8];
+        uint4 v[8];
 #pragma unroll
         for (int k = 0; k < 8; ++k)
-          if (k0 + k < K) {
-            const float* row = y + (static_cast<size_t>(t) * K + k0 + k) * H;
-            v[k] = ld16(row + c);
-            if (has2) u[k] = ld16(row + c2);
-          }
+          if (k0 + k < K) v[k] = ld16(yrow + static_cast<size_t>(k0 + k) * H + c);
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < 8; ++k)
           if (k0 + k < K && ((valid >> (k0 + k)) & 1u)) {
-            s0.x += __uint_as_float(v[k].x);
-            s0.y += __uint_as_float(v[k].y);
-            s0.z += __uint_as_float(v[k].z);
-            s0.w += __uint_as_float(v[k].w);
-            if (has2) {
-              s1.x += __uint_as_float(u[k].x);
-              s1.y += __uint_as_float(u[k].y);
-              s1.z += __uint_as_float(u[k].z);
-              s1.w += __uint_as_float(u[k].w);
-            }
+            float f[8];
+            unpack<BF16>(v[k], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s[i] += f[i];
           }
-        }
       }
-      unsigned lo = f2bf(s0.x) | (f2bf(s0.y) << 16), hi = f2bf(s0.z) | (f2bf(s0.w) << 16);
-      *as_global(reinterpret_cast<unsigned long long*>(out + static_cast<size_t>(t) * H + c)) =
-          static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32);
-      if (has2) {
-        lo = f2bf(s1.x) | (f2bf(s1.y) << 16);
-        hi = f2bf(s1.z) | (f2bf(s1.w) << 16);
-        *as_global(reinterpret_cast<unsigned long long*>(out + static_cast<size_t>(t) * H + c2)) =
-            static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32);
-      }
+      st16(out + static_cast<size_t>(t) * H + c,
+           u32x4{f2bf(s[0]) | (f2bf(s[1]) << 16), f2bf(s[2]) | (f2bf(s[3]) << 16),
+                 f2bf(s[4]) | (f2bf(s[5]) << 16), f2bf(s[6]) | (f2bf(s[7]) << 16)});
     }
     if ((t & 63) == 0) {
-      for (int e = threadIdx.x; e < p.E; e += T_THREADS)
-        stc(&p.masks[static_cast<size_t>(e) * p.W + (t >> 6)], 0ull);
+      for (int e = tid; e < E; e += T_THREADS) stc(&masks[static_cast<size_t>(e) * W + (t >> 6)], 0ull);
     }
   }
+  __syncthreads();  // flag[] is reused by the next task
 }
 
 // ---------------------------------------------------------------- worker loop
