@@ -275,11 +275,13 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
   return hipSuccess;
 }
 
-// The tiled variant needs bf16, tile-aligned shapes and a batch its scan tables
-// can hold; AUTO takes it once an expert sees about 48 rows on average.
+// The tiled variant needs bf16, tile-aligned shapes and token rows it can
+// address with 32-bit byte offsets; AUTO takes it once an expert sees about 48
+// rows on average.
 static bool tiled_eligible(const FlashMoeLayerDesc& d, int tokens_num) {
   return d.dtype == FLASH_MOE_BF16 && d.hidden % 256 == 0 && d.intermediate % 128 == 0 &&
-         tokens_num <= fmoe::tiled_max_tokens();
+         tokens_num <= fmoe::tiled_max_tokens() &&
+         static_cast<long long>(tokens_num) * d.hidden * 2 < (1ll << 32);
 }
 
 int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num) {

@@ -44,6 +44,7 @@ struct Control {
   ControlLine launches;     // completed launches (diagnostic)
   ControlLine xq[8];        // tiled variant: per-XCD ticket counters of the GEMM tasks
   ControlLine cticket;      // tiled variant: combine tickets
+  ControlLine scan_done;    // tiled variant: per-expert scan tasks finished
 };
 
 // Phase flags, one line per workgroup: the worker that completes a phase

@@ -229,55 +229,48 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
 }
 
 // ----------------------------------------------------------------------- scan
-// Same tables as the streaming variant's scan, computed by one workgroup:
-// thread e walks expert e's mask words (their popcounts were gathered into LDS
-// by all threads first), then one wave scans over the experts.
+// Same tables as the streaming variant's scan, in two steps. Expert scan: one
+// wave per expert walks the expert's mask words 64 at a time and writes the
+// running count in front of every word (word_prefix) and the expert's total.
+// Final scan: one wave turns the totals into row offsets and the row-tile table.
+constexpr int SCAN_EXPERTS = T_THREADS / 64;  // experts per expert-scan task
+
+__device__ __noinline__ void tiled_expert_scan_task(const Params& p, int blk) {
+  const int E = uni(p.E), W = uni(p.W), T = uni(p.T);
+  const unsigned long long* masks = uni(p.masks);
+  int* word_prefix = uni(p.word_prefix);
+  int* expert_count = uni(p.expert_count);
+  const int lane = threadIdx.x & 63;
+  const int e = uni(blk) * SCAN_EXPERTS + uni(threadIdx.x >> 6);
+  if (e >= E) return;
+  const int wact = (T + 63) >> 6;
+  int base = 0;
+  for (int w0 = 0; w0 < wact; w0 += 64) {
+    const int w = w0 + lane;
+    const int c = w < wact ? __popcll(ldc(&masks[static_cast<size_t>(e) * W + w])) : 0;
+    const int incl = wave_inclusive_scan(c);
+    if (w < wact) stc(&word_prefix[static_cast<size_t>(e) * W + w], base + incl - c);
+    base += __shfl(incl, 63, 64);
+  }
+  if (lane == 0) stc(&expert_count[e], base);
+}
+
 __device__ __noinline__ void tiled_scan_task(const Params& p) {
   const RouteTables r = route_tables(p);
   const int tid = threadIdx.x;
-  const int wact = (r.T + 63) >> 6;
-  unsigned char* pc = lds_raw;                                       // [E][wact] popcounts
-  int* cnt = reinterpret_cast<int*>(lds_raw + ((MAX_EXPERTS * wact + 15) & ~15));  // [E]
-  const int total = r.E * wact;
-  for (int i0 = tid; i0 < total; i0 += T_THREADS * 8) {
-    unsigned long long m[8];
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      const int i = i0 + b * T_THREADS;
-      m[b] = 0ull;
-      if (i < total) m[b] = ldc(&r.masks[static_cast<size_t>(i / wact) * r.W + (i % wact)]);
-    }
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      const int i = i0 + b * T_THREADS;
-      if (i < total) pc[i] = static_cast<unsigned char>(__popcll(m[b]));
-    }
-  }
-  __syncthreads();
-  if (tid < r.E) {
-    int c = 0;
-    int* wp = r.word_prefix + static_cast<size_t>(tid) * r.W;
-    for (int w = 0; w < wact; ++w) {
-      stc(&wp[w], c);
-      c += pc[tid * wact + w];
-    }
-    cnt[tid] = c;
-  }
-  __syncthreads();
   if (tid < 64) {
     const int lane = tid;
     const int epl = (r.E + 63) >> 6;
     int base = 0, tile_base = 0;
     for (int j = 0; j < epl; ++j) {
       const int e = lane + 64 * j;
-      const int c = e < r.E ? cnt[e] : 0;
+      const int c = e < r.E ? ldc(&r.expert_count[e]) : 0;
       const int incl = wave_inclusive_scan(c);
       const int off = base + incl - c;
       const int nt = (c + TM - 1) / TM;
       const int tincl = wave_inclusive_scan(nt);
       const int toff = tile_base + tincl - nt;
       if (e < r.E) {
-        stc(&r.expert_count[e], c);
         stc(&r.expert_offset[e], off);
         for (int i = 0; i < nt; ++i) {
           if (toff + i < r.max_mtiles) {
@@ -802,8 +795,10 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
   Control* ctl = p.ctl;
   const unsigned T = static_cast<unsigned>(p.T);
   const unsigned n_rt = (T + RT_TOK - 1u) / RT_TOK;
-  const unsigned t_scan = n_rt;
-  const unsigned t_scatter0 = n_rt + 1u;
+  const unsigned n_es = (static_cast<unsigned>(p.E) + SCAN_EXPERTS - 1u) / SCAN_EXPERTS;
+  const unsigned t_escan0 = n_rt;
+  const unsigned t_scan = n_rt + n_es;
+  const unsigned t_scatter0 = t_scan + 1u;
   const unsigned t_dyn0 = t_scatter0 + n_rt;
   const unsigned nt1 = static_cast<unsigned>(p.I / G1_COLS);
   const unsigned nt2 = static_cast<unsigned>(p.H / TN);
@@ -840,8 +835,16 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
       tiled_router_task(p, static_cast<int>(tk));
       wg_arrive<false>(&ctl->router_done.v, &sh);
       trace(tk, 0, tk, t_fetch, t_ready);
-    } else if (tk == t_scan) {
+    } else if (tk < t_scan) {
       ok = wg_wait_ge(p, &ctl->router_done.v, n_rt, &sh);
+      if (ok) {
+        if (p.trace) t_ready = wall_clock64();
+        tiled_expert_scan_task(p, static_cast<int>(tk - t_escan0));
+        wg_arrive<false>(&ctl->scan_done.v, &sh);
+        trace(tk, 6, tk - t_escan0, t_fetch, t_ready);
+      }
+    } else if (tk == t_scan) {
+      ok = wg_wait_ge(p, &ctl->scan_done.v, n_es, &sh);
       if (ok) {
         if (p.trace) t_ready = wall_clock64();
         tiled_scan_task(p);
@@ -936,13 +939,14 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
       stc(&ctl->n_mtiles.v, 0u);
       stc(&ctl->exit_count.v, 0u);
       stc(&ctl->cticket.v, 0u);
+      stc(&ctl->scan_done.v, 0u);
       stc(&ctl->ticket.v, 0u);
     }
   }
 }
 
-// Largest token count the scan task's LDS tables allow.
-int tiled_max_tokens() { return ((TILED_LDS_BYTES - 2048) / MAX_EXPERTS) * 64; }
+// Largest token count of the tiled variant: the launcher's capacity at top-1.
+int tiled_max_tokens() { return 1 << 21; }
 
 hipError_t launch_tiled_kernel(const Params& p, int grid, hipStream_t stream) {
   hipLaunchKernelGGL(moe_tiled_kernel, dim3(grid), dim3(T_THREADS), TILED_LDS_BYTES, stream, p);
