@@ -80,6 +80,13 @@ __device__ __forceinline__ void stc16(void* p, const uint4& v) {
   stc(q, static_cast<unsigned long long>(v.x) | (static_cast<unsigned long long>(v.y) << 32));
   stc(q + 1, static_cast<unsigned long long>(v.z) | (static_cast<unsigned long long>(v.w) << 32));
 }
+// 16 bytes written through to device-coherent memory (agent scope): visible to
+// every XCD once the store has completed, with no cache write-back needed.
+__device__ __forceinline__ void st16_through(void* p, const uint4& v) {
+  typedef unsigned v4u __attribute__((ext_vector_type(4)));
+  const v4u d = {v.x, v.y, v.z, v.w};
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(d) : "memory");
+}
 __device__ __forceinline__ TileDesc ld_tile(const TileDesc* t) {
   const uint4 v = ldc16(t);
   TileDesc d;

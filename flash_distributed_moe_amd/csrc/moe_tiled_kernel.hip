@@ -104,13 +104,12 @@ __device__ __forceinline__ bool wg_wait_flag(const Params& p, int which, WgShare
   return ok;
 }
 
-// All threads' stores have completed, then one thread bumps the counter.
-// WRITEBACK: the task wrote tile data (h, y) with ordinary cached stores, so the
-// XCD's L2 is written back to memory first (one agent-scope release per task and
-// workgroup is cheap; per wave task it is not, which is why the streaming
-// variant writes through instead). Readers of h and y use ordinary loads: every
-// cache line of them has a single writer and is not read before it is final,
-// so no reader can hold a stale copy.
+// All threads' stores have completed, then one thread bumps the counter. Tile
+// data (h, y) is written through to device-coherent memory, so completion is
+// all a reader on another XCD needs (WRITEBACK adds an agent-scope release for
+// data written with ordinary cached stores; no task does that at present).
+// Readers of h and y use ordinary loads: every cache line of them has a single
+// writer and is not read before it is final, so no reader can hold a stale copy.
 template <bool WRITEBACK>
 __device__ __forceinline__ unsigned wg_arrive(unsigned* counter, WgShared* sh) {
   fence_release();
@@ -352,6 +351,7 @@ __device__ __forceinline__ void load_to_lds(unsigned off, const unsigned char* b
 
 #ifdef FMOE_DBG_STALL  // timing experiment: cycles a wave spends in the load wait and in the barrier
 __device__ unsigned long long g_stall[4];
+__shared__ unsigned sh_stall[4];  // last tile loop of wave 0: load wait, barrier, whole loop (cycles)
 __device__ __forceinline__ unsigned long long stall_clock() {
   const unsigned long long t = __builtin_amdgcn_s_memtime();
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -518,6 +518,11 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   step(ks++, I0{}, std::false_type{}, std::false_type{});
   step(ks, I0{}, std::false_type{}, std::true_type{});
 #ifdef FMOE_DBG_STALL
+  if (threadIdx.x == 0) {
+    sh_stall[0] = static_cast<unsigned>(stall_vm);
+    sh_stall[1] = static_cast<unsigned>(stall_bar);
+    sh_stall[2] = static_cast<unsigned>(stall_clock() - loop_c0);
+  }
   if (lane == 0) {
     atomicAdd(&g_stall[0], stall_vm);
     atomicAdd(&g_stall[1], stall_bar);
@@ -620,7 +625,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
         const int trow = tok0 + j * 32 + rr;
         const uint4 v = *reinterpret_cast<const uint4*>(slab + rr * SLD + cc);
         if (trow < tile.rows)
-          st16(h + static_cast<size_t>(trow) * I + cc, u32x4{v.x, v.y, v.z, v.w});
+          st16_through(h + static_cast<size_t>(trow) * I + cc, v);
       }
       lds_wave_sync();
     }
@@ -710,7 +715,7 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
         const int d3 = __builtin_amdgcn_readlane(dstrow[j], it * 4 + 3);
         const int dst = q == 0 ? d0 : q == 1 ? d1 : q == 2 ? d2 : d3;
         const uint4 v = *reinterpret_cast<const uint4*>(slab + (it * 4 + q) * SLD + (lane & 15) * 8);
-        if (dst >= 0) st16(y + static_cast<size_t>(dst) * H, u32x4{v.x, v.y, v.z, v.w});
+        if (dst >= 0) st16_through(y + static_cast<size_t>(dst) * H, v);
       }
       lds_wave_sync();
     }
@@ -815,8 +820,13 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
       st16(reinterpret_cast<char*>(r) + 16,
            u32x4{static_cast<unsigned>(t_fetch), static_cast<unsigned>(t_fetch >> 32),
                  static_cast<unsigned>(t_ready), static_cast<unsigned>(t_ready >> 32)});
+#ifdef FMOE_DBG_STALL
+      const unsigned x0 = (sh_stall[0] >> 4) | ((sh_stall[1] >> 4) << 16), x1 = sh_stall[2];
+#else
+      const unsigned x0 = 0u, x1 = 0u;
+#endif
       st16(reinterpret_cast<char*>(r) + 32,
-           u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), 0u, 0u});
+           u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), x0, x1});
     }
   };
 
@@ -887,7 +897,7 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
         if (p.trace) t_ready = wall_clock64();
         const TileDesc tile = ld_tile(&p.mtiles[m]);
         tiled_gateup_task(p, tile, static_cast<int>(j % nt1));
-        wg_arrive<true>(&p.g1_done[m].v, &sh);
+        wg_arrive<false>(&p.g1_done[m].v, &sh);
         trace(t_dyn0 + lo * nt1 + j, 3, m, t_fetch, t_ready);
       } else {
         const unsigned jj = j - q1;
@@ -897,7 +907,7 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
           if (p.trace) t_ready = wall_clock64();
           const TileDesc tile = ld_tile(&p.mtiles[m]);
           tiled_down_task(p, tile, static_cast<int>(jj % nt2));
-          if (wg_arrive<true>(&ctl->g2_done.v, &sh) == n2_total - 1u) wg_broadcast_flag(p, FLAG_G2);
+          if (wg_arrive<false>(&ctl->g2_done.v, &sh) == n2_total - 1u) wg_broadcast_flag(p, FLAG_G2);
           trace(t_dyn0 + nm * nt1 + lo * nt2 + jj, 4, m, t_fetch, t_ready);
         }
       }

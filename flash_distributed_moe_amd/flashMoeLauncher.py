@@ -159,7 +159,7 @@ class MoeKernelLauncher:
 
     TRACE_DTYPE = np.dtype([("ticket", "<u4"), ("kind", "<u4"), ("worker", "<u4"), ("aux", "<u4"),
                             ("t_fetch", "<i8"), ("t_ready", "<i8"), ("t_end", "<i8"),
-                            ("pad", "<i8")])
+                            ("x0", "<u4"), ("x1", "<u4")])  # spare words (timing experiments)
 
     def trace_enable(self, capacity):
         _hip_check(self._lib.flashMoeTraceEnable(self._h, int(capacity)), "flashMoeTraceEnable")
