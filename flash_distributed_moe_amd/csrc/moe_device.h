@@ -188,6 +188,14 @@ __device__ __forceinline__ unsigned f2bf(float f) {
   return u >> 16;
 }
 
+// two floats to packed bf16 (round to nearest even) with the hardware converter
+__device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  const f2 v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf2));
+}
+
 template <typename DT>
 __device__ __forceinline__ void unpack(const uint4& v, float (&f)[DT::EPV]);
 template <>
@@ -481,6 +489,14 @@ __device__ __forceinline__ float silu_mul(float a, float b) {
     const float e = __expf(a);
     s = e / (1.0f + e);
   }
+  return a * s * b;
+}
+// The same function with the hardware reciprocal (1 ulp) in place of the
+// division: e = exp(-|a|), sigmoid = (a >= 0 ? 1 : e) / (1 + e).
+__device__ __forceinline__ float silu_mul_fast(float a, float b) {
+  const float e = __expf(-__builtin_fabsf(a));
+  const float r = __builtin_amdgcn_rcpf(1.0f + e);
+  const float s = a >= 0.0f ? r : e * r;
   return a * s * b;
 }
 

@@ -612,10 +612,10 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
           float hv[4];
 #pragma unroll
           for (int v = 0; v < 4; ++v)
-            hv[v] = silu_mul(acc[i][j][g4 * 4 + v], acc[i + 2][j][g4 * 4 + v]);
+            hv[v] = silu_mul_fast(acc[i][j][g4 * 4 + v], acc[i + 2][j][g4 * 4 + v]);
           uint2 pk;
-          pk.x = f2bf(hv[0]) | (f2bf(hv[1]) << 16);
-          pk.y = f2bf(hv[2]) | (f2bf(hv[3]) << 16);
+          pk.x = pack_bf16(hv[0], hv[1]);
+          pk.y = pack_bf16(hv[2], hv[3]);
           *reinterpret_cast<uint2*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) = pk;
         }
       lds_wave_sync();
@@ -700,8 +700,8 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           uint2 pk;
-          pk.x = f2bf(acc[i][j][g4 * 4 + 0] * w) | (f2bf(acc[i][j][g4 * 4 + 1] * w) << 16);
-          pk.y = f2bf(acc[i][j][g4 * 4 + 2] * w) | (f2bf(acc[i][j][g4 * 4 + 3] * w) << 16);
+          pk.x = pack_bf16(acc[i][j][g4 * 4 + 0] * w, acc[i][j][g4 * 4 + 1] * w);
+          pk.y = pack_bf16(acc[i][j][g4 * 4 + 2] * w, acc[i][j][g4 * 4 + 3] * w);
           *reinterpret_cast<uint2*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) = pk;
         }
       lds_wave_sync();
@@ -763,8 +763,8 @@ __device__ __noinline__ void tiled_combine_task(const Params& p, int blk) {
           }
       }
       st16(out + static_cast<size_t>(t) * H + c,
-           u32x4{f2bf(s[0]) | (f2bf(s[1]) << 16), f2bf(s[2]) | (f2bf(s[3]) << 16),
-                 f2bf(s[4]) | (f2bf(s[5]) << 16), f2bf(s[6]) | (f2bf(s[7]) << 16)});
+           u32x4{pack_bf16(s[0], s[1]), pack_bf16(s[2], s[3]), pack_bf16(s[4], s[5]),
+                 pack_bf16(s[6], s[7])});
     }
     if ((t & 63) == 0) {
       for (int e = tid; e < E; e += T_THREADS) stc(&masks[static_cast<size_t>(e) * W + (t >> 6)], 0ull);
