@@ -36,13 +36,16 @@ constexpr int TN = 256;            // weight rows per tile
 constexpr int TK = 32;             // k per LDS stage (one 64-byte row slice)
 constexpr int STAGES = 4;          // LDS stages in flight
 constexpr int STAGE_BYTES = (TM + TN) * TK * 2;  // 32 KiB: weight rows, then token rows
-constexpr int T_THREADS = 256;
+constexpr int T_THREADS = 512;
+constexpr int WAVES = T_THREADS / 64;  // two per SIMD: one wave's loads and LDS reads hide behind the other's MFMAs
+constexpr int WJ = 16 / WAVES;         // 32-row token blocks per wave (each wave: 128 weight rows x 32*WJ token rows)
+constexpr int LQ = 16 / WAVES;         // 16-row loads per operand, stage and wave
 constexpr int G1_COLS = TN / 2;    // h columns per gate/up task
 constexpr int RT_TOK = 32;         // tokens per router / scatter task
 constexpr int CMB_TOK = 8;         // tokens per combine task
 
 constexpr int TILE_LDS_BYTES = STAGES * STAGE_BYTES;  // 131072
-constexpr int ROUTER_LDS_BYTES = RT_TOK * MAX_EXPERTS * 4 + 4 * MAX_TOPK * 8;
+constexpr int ROUTER_LDS_BYTES = RT_TOK * MAX_EXPERTS * 4 + WAVES * MAX_TOPK * 8;
 constexpr int TILED_LDS_BYTES = TILE_LDS_BYTES > ROUTER_LDS_BYTES ? TILE_LDS_BYTES : ROUTER_LDS_BYTES;
 
 extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -145,7 +148,7 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
   const unsigned short* gate = uni(reinterpret_cast<const unsigned short*>(p.gate));
   const float* bias = uni(p.bias);
   unsigned* keys = reinterpret_cast<unsigned*>(lds_raw);  // [RT_TOK][MAX_EXPERTS] ordered logits
-  double* sel = reinterpret_cast<double*>(keys + RT_TOK * MAX_EXPERTS);  // 4 waves x MAX_TOPK
+  double* sel = reinterpret_cast<double*>(keys + RT_TOK * MAX_EXPERTS);  // WAVES x MAX_TOPK
   const int tid = threadIdx.x;
   const int wave = uni(tid >> 6), lane = tid & 63;
   const int th = wave >> 1, eh = wave & 1;
@@ -154,7 +157,8 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
   const unsigned short* xrow =
       tokens + static_cast<size_t>(min(t0 + th * 16 + l16, T - 1)) * H;
 
-  for (int e0 = 0; e0 < E; e0 += 128) {
+  // the chain keeps one wave per SIMD busy: waves 0..3 (token half, expert half)
+  for (int e0 = 0; e0 < E && wave < 4; e0 += 128) {
     const unsigned short* wrow =
         gate + static_cast<size_t>(min(e0 + eh * 64 + lane, E - 1)) * H;
     f32x16 acc;
@@ -210,10 +214,10 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
     }
   }
   __syncthreads();
-  // selection: each wave takes 8 of the 32 tokens
+  // selection: the tokens are dealt out over all waves
   double* lex = sel + wave * MAX_TOPK;
-  for (int i = 0; i < RT_TOK / 4; ++i) {
-    const int tl = wave * (RT_TOK / 4) + i;
+  for (int i = 0; i < RT_TOK / WAVES; ++i) {
+    const int tl = wave * (RT_TOK / WAVES) + i;
     const int t = t0 + tl;
     if (t < T) {
       unsigned val[MAX_EXPERTS / 64];
@@ -319,8 +323,8 @@ __device__ void tiled_scatter_task(const Params& p, int blk) {
 struct TileRows {
   const unsigned char* wbase;  // uniform: expert's weight matrix
   const unsigned char* tbase;  // uniform: tokens, or this tile's h rows
-  unsigned woff[4];            // byte offset of this lane's chunk of weight-stage row wave*64+q*16+(lane>>2)
-  unsigned toff[4];            // same for the token stage
+  unsigned woff[LQ];           // byte offset of this lane's chunk of weight-stage row wave*16*LQ+q*16+(lane>>2)
+  unsigned toff[LQ];           // same for the token stage
 };
 
 #define FMOE_G1 __attribute__((address_space(1)))
@@ -360,17 +364,18 @@ __device__ __forceinline__ unsigned long long stall_clock() {
 #endif
 
 struct Frags {
-  uint4 a[4];  // weight blocks
-  uint4 b[4];  // token blocks
+  uint4 a[4];   // weight blocks
+  uint4 b[WJ];  // token blocks
 };
 
-// Interleave hint for one half k-step: one LDS read, then two matrix
-// instructions, eight times over.
+// Interleave hint for one half k-step: the 4 + WJ LDS reads spread evenly
+// between the 4 * WJ matrix instructions.
 __device__ __forceinline__ void interleave_reads_and_mfma() {
+  constexpr int PER = (4 * WJ) / (4 + WJ);
 #pragma unroll
-  for (int n = 0; n < 8; ++n) {
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+  for (int n = 0; n < 4 + WJ; ++n) {
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // DS read
+    __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // MFMA
   }
 }
 
@@ -380,32 +385,32 @@ __device__ __forceinline__ void interleave_reads_and_mfma() {
 // Every wave loads its share of each stage whatever its JMAX.
 template <int JMAX>
 __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, const int (&wblk)[4],
-                                            int tok0, f32x16 (&acc)[4][4]) {
+                                            int tok0, f32x16 (&acc)[4][WJ]) {
   const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
   const int r32 = lane & 31, kq = lane >> 5;
   const unsigned char* lds = lds_raw;
   const unsigned lds_addr = uni(static_cast<unsigned>(
       reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
 
-  // load q (0..3: weight rows, 4..7: token rows) of this wave's 8 loads of
-  // k-step ks into stage ks % STAGES
+  // load q (0..LQ-1: weight rows, LQ..2*LQ-1: token rows) of this wave's loads
+  // of k-step ks into stage ks % STAGES
   auto issue_one = [&](int ks, int q) {
 #ifdef FMOE_DBG_NO_GLOBAL  // timing experiment: keep re-reading the first k-steps (cache hits)
     const int src = ks & 3;
 #else
     const int src = ks;
 #endif
-    const unsigned st = lds_addr + (ks & (STAGES - 1)) * STAGE_BYTES + wave * 4096;
-    if (q < 4) {
+    const unsigned st = lds_addr + (ks & (STAGES - 1)) * STAGE_BYTES + wave * (LQ * 1024);
+    if (q < LQ) {
       load_to_lds(rows.woff[q], rows.wbase + static_cast<size_t>(src) * (TK * 2), st + q * 1024);
     } else {
-      load_to_lds(rows.toff[q - 4], rows.tbase + static_cast<size_t>(src) * (TK * 2),
-                  st + TN * TK * 2 + (q - 4) * 1024);
+      load_to_lds(rows.toff[q - LQ], rows.tbase + static_cast<size_t>(src) * (TK * 2),
+                  st + TN * TK * 2 + (q - LQ) * 1024);
     }
   };
   auto issue = [&](int ks) {
 #pragma unroll
-    for (int q = 0; q < 8; ++q) issue_one(ks, q);
+    for (int q = 0; q < 2 * LQ; ++q) issue_one(ks, q);
   };
 
   // per-lane read offsets: row r32 of a block, chunk kk*2+kq at its permuted position
@@ -425,7 +430,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
 #pragma unroll
     for (int i = 0; i < 4; ++i) read_a(f, ks, kk, i);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) read_b(f, ks, kk, j);
+    for (int j = 0; j < WJ; ++j) read_b(f, ks, kk, j);
   };
   auto mfma_block = [&](const Frags& f, int j) {
     if (j < JMAX) {
@@ -445,7 +450,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   // the next stage is confirmed, the stage just finished is refilled, and the
   // next step's first half is read — loads and reads spread between the matrix
   // instructions. PENDING: loads of later stages that may still be in flight
-  // when stage ks+1 has to be complete (8 per stage).
+  // when stage ks+1 has to be complete (2 * LQ per stage).
   Frags f0, f1;
 #ifdef FMOE_DBG_STALL
   unsigned long long stall_vm = 0, stall_bar = 0;
@@ -461,7 +466,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
     if (ks == 0) read(f1, ks, 1);
 #endif
 #pragma unroll
-    for (int j = 0; j < 4; ++j) mfma_block(f0, j);
+    for (int j = 0; j < WJ; ++j) mfma_block(f0, j);
     interleave_reads_and_mfma();
     __builtin_amdgcn_sched_barrier(0);
     if (!LAST) {
@@ -481,7 +486,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
       stall_bar += c2 - c1;
 #endif
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int g = 0; g < WJ; ++g) {
         mfma_block(f1, g);
         __builtin_amdgcn_sched_barrier(0);
 #ifndef FMOE_DBG_NO_REFILL  // timing experiment: the main loop issues no loads
@@ -491,23 +496,24 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
         }
 #endif
 #ifndef FMOE_DBG_NO_READS  // timing experiment: the main loop reads no fragments
-        read_a(f0, ks + 1, 0, g);
+#pragma unroll
+        for (int i = g * (4 / WJ); i < (g + 1) * (4 / WJ); ++i) read_a(f0, ks + 1, 0, i);
         read_b(f0, ks + 1, 0, g);
 #endif
         __builtin_amdgcn_sched_barrier(0);
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) mfma_block(f1, j);
+      for (int j = 0; j < WJ; ++j) mfma_block(f1, j);
     }
   };
   using I0 = std::integral_constant<int, 0>;
-  using I8 = std::integral_constant<int, 8>;
-  using I16 = std::integral_constant<int, 16>;
+  using I8 = std::integral_constant<int, 2 * LQ>;   // one later stage in flight
+  using I16 = std::integral_constant<int, 4 * LQ>;  // two later stages in flight
 
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) issue(s);  // ksteps >= STAGES for every admitted shape
-  wait_vm<24>();
+  wait_vm<6 * LQ>();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   read(f0, 0, 0);
@@ -537,20 +543,20 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
 // Rounding it up is safe: rows past the tile's end are clamped copies whose
 // results the epilogue drops.
 __device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, const int (&wblk)[4],
-                                          int tok0, int jmax, f32x16 (&acc)[4][4]) {
-  if (jmax > 2) {
-    tile_gemm_j<4>(rows, ksteps, wblk, tok0, acc);
+                                          int tok0, int jmax, f32x16 (&acc)[4][WJ]) {
+  if (jmax > WJ / 2) {
+    tile_gemm_j<WJ>(rows, ksteps, wblk, tok0, acc);
   } else if (jmax > 0) {
-    tile_gemm_j<2>(rows, ksteps, wblk, tok0, acc);
+    tile_gemm_j<WJ / 2>(rows, ksteps, wblk, tok0, acc);
   } else {
     tile_gemm_j<0>(rows, ksteps, wblk, tok0, acc);
   }
 }
 
-// The chunk lane `lane` of wave `wave` loads for stage row wave*64 + q*16 + (lane >> 2):
+// The chunk lane `lane` of wave `wave` loads for stage row wave*16*LQ + q*16 + (lane >> 2):
 // position lane & 3 of that row holds chunk (lane & 3) ^ ((row >> 2) & 3).
 __device__ __forceinline__ int stage_row(int q) {
-  return (threadIdx.x >> 6) * 64 + q * 16 + ((threadIdx.x & 63) >> 2);
+  return (threadIdx.x >> 6) * (16 * LQ) + q * 16 + ((threadIdx.x & 63) >> 2);
 }
 __device__ __forceinline__ unsigned stage_chunk_bytes(int row) {
   return static_cast<unsigned>(((threadIdx.x & 3) ^ ((row >> 2) & 3)) << 4);
@@ -571,7 +577,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
   rows.wbase = reinterpret_cast<const unsigned char*>(w13);
   rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
+  for (int q = 0; q < LQ; ++q) {
     const int row = stage_row(q);
     // weight stage rows 0..127: gate rows n0+row, 128..255: up rows I+n0+(row-128)
     const int wrow = row < G1_COLS ? n0 + row : I + n0 + (row - G1_COLS);
@@ -582,15 +588,15 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
   const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int wn = wave & 1, wm = wave >> 1;
   const int wblk[4] = {wn * 64, wn * 64 + 32, G1_COLS + wn * 64, G1_COLS + wn * 64 + 32};
-  const int tok0 = wm * 128;
-  const int jmax = uni(min(4, max(0, (tile.rows - tok0 + 31) / 32)));
+  const int tok0 = wm * (32 * WJ);
+  const int jmax = uni(min(WJ, max(0, (tile.rows - tok0 + 31) / 32)));
   unsigned short* h = uni(reinterpret_cast<unsigned short*>(p.h)) +
                       static_cast<size_t>(tile.row0) * I + n0 + wn * 64;
-  f32x16 acc[4][4];
+  f32x16 acc[4][WJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < WJ; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
@@ -603,7 +609,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
   constexpr int SLD = 64 + 8;  // slab row stride, bf16 elements
   unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * 32 * SLD;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < WJ; ++j) {
     if (j < jmax) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
@@ -648,7 +654,7 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
   rows.tbase = reinterpret_cast<const unsigned char*>(
       uni(reinterpret_cast<const unsigned short*>(p.h)) + static_cast<size_t>(tile.row0) * I);
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
+  for (int q = 0; q < LQ; ++q) {
     const int row = stage_row(q);
     rows.woff[q] = static_cast<unsigned>(n0 + row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
     rows.toff[q] = static_cast<unsigned>(min(row, tile.rows - 1)) * static_cast<unsigned>(I * 2) +
@@ -657,30 +663,30 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
   const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int wn = wave & 1, wm = wave >> 1;
   const int wblk[4] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
-  const int tok0 = wm * 128;
-  const int jmax = uni(min(4, max(0, (tile.rows - tok0 + 31) / 32)));
+  const int tok0 = wm * (32 * WJ);
+  const int jmax = uni(min(WJ, max(0, (tile.rows - tok0 + 31) / 32)));
   const int r32 = lane & 31, kq = lane >> 5;
   // y rows are bf16 here: H values per (token, slot)
   unsigned short* y = uni(reinterpret_cast<unsigned short*>(p.y)) + n0 + wn * 128 + (lane & 15) * 8;
   // gate weight and destination row (token*K + slot) of this lane's row in each token block
-  float roww[4];
-  int dstrow[4];
+  float roww[WJ];
+  int dstrow[WJ];
   {
     const float* row_w = uni(p.row_w) + tile.row0;
     const int* perm = uni(p.perm) + tile.row0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < WJ; ++j) {
       const int myrow = tok0 + j * 32 + r32;
       const bool valid = myrow < tile.rows;
       roww[j] = valid ? ldc(&row_w[myrow]) : 0.0f;
       dstrow[j] = valid ? ldc(&perm[myrow]) : -1;
     }
   }
-  f32x16 acc[4][4];
+  f32x16 acc[4][WJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < WJ; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
@@ -692,7 +698,7 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
   constexpr int SLD = 128 + 8;  // slab row stride, bf16 elements
   unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * (32 * SLD);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < WJ; ++j) {
     if (j < jmax) {
       const float w = roww[j];
 #pragma unroll
@@ -737,35 +743,37 @@ __device__ __noinline__ void tiled_combine_task(const Params& p, int blk) {
   unsigned char* flag = lds_raw;  // [CMB_TOK * MAX_TOPK]
   if (tid < ntok * K) flag[tid] = ldc(&topk_idx[static_cast<size_t>(t0) * K + tid]) >= 0 ? 1 : 0;
   __syncthreads();
-  for (int tl = 0; tl < ntok; ++tl) {
+  // one item = 8 columns of one token; the K row loads of an item are in flight together
+  const int cpr = H >> 3;  // items per token
+  for (int it = tid; it < ntok * cpr; it += T_THREADS) {
+    const int tl = it / cpr, c = (it - tl * cpr) << 3;
     const int t = t0 + tl;
     unsigned valid = 0u;
     for (int k = 0; k < K; ++k) valid |= static_cast<unsigned>(flag[tl * K + k]) << k;
-    valid = uni(static_cast<int>(valid));
-    const unsigned short* yrow = y + static_cast<size_t>(t) * K * H;
-    // 8 columns per thread and pass; the K row loads of a pass are in flight together
-    for (int c = tid * 8; c < H; c += T_THREADS * 8) {
-      float s[8];
+    const unsigned short* yrow = y + static_cast<size_t>(t) * K * H + c;
+    float s[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) s[i] = 0.0f;
-      for (int k0 = 0; k0 < K; k0 += 8) {
-        uint4 v[8];
+    for (int i = 0; i < 8; ++i) s[i] = 0.0f;
+    for (int k0 = 0; k0 < K; k0 += 8) {
+      uint4 v[8];
 #pragma unroll
-        for (int k = 0; k < 8; ++k)
-          if (k0 + k < K) v[k] = ld16(yrow + static_cast<size_t>(k0 + k) * H + c);
+      for (int k = 0; k < 8; ++k)
+        if (k0 + k < K) v[k] = ld16(yrow + static_cast<size_t>(k0 + k) * H);
 #pragma unroll
-        for (int k = 0; k < 8; ++k)
-          if (k0 + k < K && ((valid >> (k0 + k)) & 1u)) {
-            float f[8];
-            unpack<BF16>(v[k], f);
+      for (int k = 0; k < 8; ++k)
+        if (k0 + k < K && ((valid >> (k0 + k)) & 1u)) {
+          float f[8];
+          unpack<BF16>(v[k], f);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) s[i] += f[i];
-          }
-      }
-      st16(out + static_cast<size_t>(t) * H + c,
-           u32x4{pack_bf16(s[0], s[1]), pack_bf16(s[2], s[3]), pack_bf16(s[4], s[5]),
-                 pack_bf16(s[6], s[7])});
+          for (int i = 0; i < 8; ++i) s[i] += f[i];
+        }
     }
+    st16(out + static_cast<size_t>(t) * H + c,
+         u32x4{pack_bf16(s[0], s[1]), pack_bf16(s[2], s[3]), pack_bf16(s[4], s[5]),
+               pack_bf16(s[6], s[7])});
+  }
+  for (int tl = 0; tl < ntok; ++tl) {
+    const int t = t0 + tl;
     if ((t & 63) == 0) {
       for (int e = tid; e < E; e += T_THREADS) stc(&masks[static_cast<size_t>(e) * W + (t >> 6)], 0ull);
     }
