@@ -194,15 +194,15 @@ __device__ __noinline__ void router_dot_task(const Params& p, int tg, int eg) {
 __device__ __noinline__ void router_select_task(const Params& p, int t) {
   constexpr int MAXEPL = MAX_EXPERTS / 64;
   const int lane = lane_id();
-  unsigned long long key[MAXEPL];
+  unsigned val[MAXEPL];  // the ordered logit bits are the upper half of a candidate key
 #pragma unroll
   for (int j = 0; j < MAXEPL; ++j) {
     const int e = lane + 64 * j;
-    key[j] = e < p.E ? ldc(&p.cand[static_cast<size_t>(t) * p.E + e]) : 0ull;
+    val[j] = e < p.E ? static_cast<unsigned>(ldc(&p.cand[static_cast<size_t>(t) * p.E + e]) >> 32) : 0u;
   }
   if (lane == 0) stc(&p.tok_arrive[t], 0u);
-  router_select(p, t, key,
-                reinterpret_cast<unsigned long long*>(lds_dyn + (threadIdx.x >> 6) * ROUTER_LDS_FLOATS));
+  router_select_max(p, t, val,
+                    reinterpret_cast<double*>(lds_dyn + (threadIdx.x >> 6) * ROUTER_LDS_FLOATS));
   wave_arrive(&p.ctl->router_done.v);
 }
 

@@ -137,12 +137,13 @@ def test_tiled_variant_forced(shape):
 
 @pytest.mark.parametrize("T", [1, 5, 16])
 def test_dense_small_batch_equals_routed(T):
-    """Batches of <= 16 tokens run gate/up for every (expert, token) pair; with
-    that turned off the routed path must give the same bits."""
+    """On request, batches of <= 16 tokens run gate/up for every (expert, token)
+    pair; the routed path (the default) must give the same bits."""
     cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=T, name="dense")
     case = GpuCase(cfg, seed=40 + T)
     try:
         x = case.inp["tokens"]
+        case.launcher.set_dense_small_batch(True)
         dense = case.run()
         case.check_routing(x, case.launcher.routing(T))
         case.check_outputs(x, dense)
