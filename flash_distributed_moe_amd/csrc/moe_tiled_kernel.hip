@@ -45,7 +45,7 @@ constexpr int RT_TOK = 32;         // tokens per router / scatter task
 constexpr int CMB_TOK = 8;         // tokens per combine task
 
 constexpr int TILE_LDS_BYTES = STAGES * STAGE_BYTES;  // 131072
-constexpr int ROUTER_LDS_BYTES = RT_TOK * MAX_EXPERTS * 4 + WAVES * MAX_TOPK * 8;
+constexpr int ROUTER_LDS_BYTES = 4 * 24576 + RT_TOK * MAX_EXPERTS * 4 + WAVES * MAX_TOPK * 8;
 constexpr int TILED_LDS_BYTES = TILE_LDS_BYTES > ROUTER_LDS_BYTES ? TILE_LDS_BYTES : ROUTER_LDS_BYTES;
 
 extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -133,87 +133,215 @@ __device__ __forceinline__ void wg_broadcast_flag(const Params& p, int which) {
   for (int g = threadIdx.x; g < n; g += blockDim.x) st_relaxed(&flags[g].f[which], 1u);
 }
 
+// ------------------------------------------------- direct-to-LDS load helpers
+#define FMOE_G1 __attribute__((address_space(1)))
+#define FMOE_L3 __attribute__((address_space(3)))
+
+__device__ __forceinline__ f32x16 mma32(const uint4& a, const uint4& b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// wait until at most N of this wave's vector-memory operations are outstanding
+// (they complete in order); nothing else is waited for
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// One wave-wide 16-byte-per-lane load from global memory straight into LDS:
+// lane l's 16 bytes from base + off land at LDS byte address lds_addr + 16*l.
+// Written as assembly so that the compiler does not order LDS reads of other
+// stages behind it; completion is tracked by hand with wait_vm.
+__device__ __forceinline__ void load_to_lds(unsigned off, const unsigned char* base, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(off), "s"(base), "s"(lds_addr)
+               : "memory");
+}
+
+#ifdef FMOE_DBG_STALL  // timing experiment: cycles a wave spends in the load wait and in the barrier
+__device__ unsigned long long g_stall[4];
+__shared__ unsigned sh_stall[4];  // last tile loop of wave 0: load wait, barrier, whole loop (cycles)
+__device__ __forceinline__ unsigned long long stall_clock() {
+  const unsigned long long t = __builtin_amdgcn_s_memtime();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  return t;
+}
+#endif
+
 // --------------------------------------------------------------------- router
 // Logits as in test/singleGPU/cpp/moe/reference/refGemm.h:21-24: one chain per
 // output, k ascending, one rounding per step. The chain runs on the matrix
-// core: V_MFMA_F32_16X16X1_4B_F32 adds exactly one product per output and
-// instruction, and a product of two bf16 values is exact in float, so every
-// step is the oracle's acc = fmaf(x, w, acc). Each wave carries 16 tokens x 64
-// experts (four 16x16 blocks that share the token operand); every lane streams
-// its own token row and its own expert row from global memory, 32 k at a time.
+// core: V_MFMA_F32_32X32X2_F32 adds its two products to the accumulator one
+// after the other in k order (checked bit for bit against a CPU fmaf chain; so
+// do 16X16X1 and 16X16X4), and a product of two bf16 values is exact in float,
+// so every step is the oracle's acc = fmaf(x, w, acc). A dependent chain of
+// these instructions runs at the matrix core's full rate (64 cycles each).
+// Waves 0..3 carry 32 tokens x 32 experts each, one wave per SIMD; waves 4..7
+// are the loaders: they bring the 32 token rows and
+// 128 expert rows in, 64 k at a time, with coalesced direct-to-LDS loads, four
+// stages deep. Stage rows are 144 bytes (128 of data, 16 of padding), so the
+// 16-byte reads of 16 rows at one k fall into different banks and every read
+// address is a per-lane base plus an immediate. (One LDS read costs a wave
+// about 22 cycles of issue whatever its width, hence 16-byte reads.)
 // Then selection as in refTopk.h:36-58 / refMoeGate.h:27-30.
+constexpr int RT_ROW_BYTES = 144;
+constexpr int RT_LOADS = 6;                       // loads per loader wave and stage
+constexpr int RT_STAGE_BYTES = 4 * RT_LOADS * 1024;  // 24 KiB
+constexpr int RT_TOK_LOADS = (RT_TOK * 9 + 63) / 64; // loads that hold token rows
+constexpr int RT_EXP_BASE = RT_TOK_LOADS * 1024;     // byte offset of the expert rows in a stage
+constexpr int RT_STAGES = 4;
+static_assert(RT_EXP_BASE + 128 * RT_ROW_BYTES <= RT_STAGE_BYTES, "router stage too small");
+
 __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
   const int T = uni(p.T), E = uni(p.E), H = uni(p.H);
-  const unsigned short* tokens = uni(reinterpret_cast<const unsigned short*>(p.tokens));
-  const unsigned short* gate = uni(reinterpret_cast<const unsigned short*>(p.gate));
+  const unsigned char* tokens = uni(reinterpret_cast<const unsigned char*>(p.tokens));
+  const unsigned char* gate = uni(reinterpret_cast<const unsigned char*>(p.gate));
   const float* bias = uni(p.bias);
-  unsigned* keys = reinterpret_cast<unsigned*>(lds_raw);  // [RT_TOK][MAX_EXPERTS] ordered logits
+  unsigned* keys = reinterpret_cast<unsigned*>(lds_raw + RT_STAGES * RT_STAGE_BYTES);  // [RT_TOK][MAX_EXPERTS] ordered logits
   double* sel = reinterpret_cast<double*>(keys + RT_TOK * MAX_EXPERTS);  // WAVES x MAX_TOPK
+  const unsigned lds_addr = uni(static_cast<unsigned>(
+      reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
   const int tid = threadIdx.x;
   const int wave = uni(tid >> 6), lane = tid & 63;
-  const int th = wave >> 1, eh = wave & 1;
+  const bool loader = wave >= 4;
   const int t0 = uni(blk) * RT_TOK;
-  const int l16 = lane & 15, lq = lane >> 4;
-  const unsigned short* xrow =
-      tokens + static_cast<size_t>(min(t0 + th * 16 + l16, T - 1)) * H;
+  const int nsteps = H >> 6;
+#ifdef FMOE_DBG_STALL
+  const unsigned long long rt_c0 = stall_clock();
+#endif
 
-  // the chain keeps one wave per SIMD busy: waves 0..3 (token half, expert half)
-  for (int e0 = 0; e0 < E && wave < 4; e0 += 128) {
-    const unsigned short* wrow =
-        gate + static_cast<size_t>(min(e0 + eh * 64 + lane, E - 1)) * H;
+  for (int e0 = 0; e0 < E; e0 += 128) {
+    // loader: load ld = 6*w + i fills the 64 16-byte slots from slot 64*ld on. Loads
+    // 0..4 hold the token rows, loads 5..23 the expert rows (from byte RT_EXP_BASE);
+    // within a region slot g is position g % 9 of row g / 9 (position 8 is padding,
+    // slots past the last row repeat it).
+    unsigned goff[RT_LOADS];
+#pragma unroll
+    for (int i = 0; i < RT_LOADS; ++i) {
+      const int ld = (wave & 3) * RT_LOADS + i;  // uniform
+      const bool tok = ld < RT_TOK_LOADS;
+      const int g = (tok ? ld : ld - RT_TOK_LOADS) * 64 + lane;
+      const int row = min(g / 9, (tok ? RT_TOK : 128) - 1);
+      const int pos = min(g % 9, 7);
+      const int grow = tok ? min(t0 + row, T - 1) : min(e0 + row, E - 1);
+      goff[i] = static_cast<unsigned>(grow) * static_cast<unsigned>(H * 2) + pos * 16;
+    }
+    auto issue = [&](int step) {
+      const int src = min(step, nsteps - 1);  // past the end: refill with the last step (never read)
+      const unsigned st = lds_addr + (step & (RT_STAGES - 1)) * RT_STAGE_BYTES +
+                          ((wave & 3) * RT_LOADS) * 1024;
+#ifdef FMOE_DBG_RT_NOLOAD  // timing experiment
+      if (step > 3) return;
+#endif
+#pragma unroll
+      for (int i = 0; i < RT_LOADS; ++i) {
+        const bool tok = (wave & 3) * RT_LOADS + i < RT_TOK_LOADS;
+        load_to_lds(goff[i], (tok ? tokens : gate) + static_cast<size_t>(src) * 128, st + i * 1024);
+      }
+    };
+    // consumer: wave w multiplies the 32 token rows with expert rows 32*w .. 32*w+31.
+    // Lane l: row l % 32 of both; V_MFMA_F32_32X32X2_F32 takes k = 2*s + l/32 from it,
+    // i.e. the low or the high half of 32-bit word s of the row: the byte permute
+    // moves that half into the upper 16 bits of a zero word, which makes the float.
+    const int r32 = lane & 31, kh = lane >> 5;
+    const unsigned pick = kh ? 0x07060C0Cu : 0x05040C0Cu;
+    const unsigned char* xptr = lds_raw + r32 * RT_ROW_BYTES;
+    const unsigned char* wptr = lds_raw + RT_EXP_BASE + ((wave & 3) * 32 + r32) * RT_ROW_BYTES;
     f32x16 acc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-    uint4 xr[4][4], wr[4][4];  // ring of four 32-k chunks, loads three chunks ahead
-    auto load = [&](int slot, int k) {
-      const int kc = min(k, H - 32);  // past the end: re-read the last chunk
+
+    // Operands of half a stage: four 16-byte chunks (8 k each) of both rows.
+    struct Half {
+      uint4 a[4], w[4];
+    };
+    auto read_half = [&](Half& h, int stage, int hf) {
+      const int so = (stage & (RT_STAGES - 1)) * RT_STAGE_BYTES + hf * 64;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        xr[slot][c] = ld16(xrow + kc + c * 8);
-        wr[slot][c] = ld16(wrow + kc + c * 8);
+        h.a[c] = *reinterpret_cast<const uint4*>(xptr + so + c * 16);
+        h.w[c] = *reinterpret_cast<const uint4*>(wptr + so + c * 16);
       }
-      __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the chain they overlap
     };
-    auto chain = [&](int slot) {
+    // The 16 MFMAs of one half, and between them the reads of another half: one pair
+    // of reads after every fourth MFMA. A read costs the wave about 20 cycles of
+    // issue, which fits in the 64 cycles the next (dependent) MFMA has to wait anyway;
+    // the scheduling barriers keep the compiler from moving the reads to the end.
+    auto chain_and_read = [&](const Half& h, Half& nx, int stage, int hf) {
+      const int so = (stage & (RT_STAGES - 1)) * RT_STAGE_BYTES + hf * 64;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const unsigned xw[4] = {xr[slot][c].x, xr[slot][c].y, xr[slot][c].z, xr[slot][c].w};
-        const unsigned ww[4] = {wr[slot][c].x, wr[slot][c].y, wr[slot][c].z, wr[slot][c].w};
+        const unsigned xw[4] = {h.a[c].x, h.a[c].y, h.a[c].z, h.a[c].w};
+        const unsigned ww[4] = {h.w[c].x, h.w[c].y, h.w[c].z, h.w[c].w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          acc = __builtin_amdgcn_mfma_f32_16x16x1f32(bf16_lo(xw[i]), bf16_lo(ww[i]), acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_16x16x1f32(bf16_hi(xw[i]), bf16_hi(ww[i]), acc, 0, 0, 0);
-        }
+        for (int m = 0; m < 4; ++m)
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(
+              __uint_as_float(__builtin_amdgcn_perm(xw[m], 0u, pick)),
+              __uint_as_float(__builtin_amdgcn_perm(ww[m], 0u, pick)), acc, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        nx.a[c] = *reinterpret_cast<const uint4*>(xptr + so + c * 16);
+        nx.w[c] = *reinterpret_cast<const uint4*>(wptr + so + c * 16);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
     };
-    load(0, 0);
-    load(1, 32);
-    load(2, 64);
-    for (int k0 = 0; k0 < H; k0 += 128) {
-      load(3, k0 + 96);
-      chain(0);
-      load(0, k0 + 128);
-      chain(1);
-      load(1, k0 + 160);
-      chain(2);
-      load(2, k0 + 192);
-      chain(3);
+
+    // Loaders and consumers run separate loops with the same number of barriers:
+    // barrier s (in the middle of step s) means "stage s+1 is in, nobody reads
+    // stage s any more".
+    if (loader) {
+      issue(0);
+      issue(1);
+      issue(2);
+      issue(3);
+      wait_vm<3 * RT_LOADS>();
+      __builtin_amdgcn_s_barrier();  // stage 0 is in
+      for (int s = 0; s < nsteps; ++s) {
+        wait_vm<2 * RT_LOADS>();  // stage s+1 is in; s+2 and s+3 may be in flight
+        __builtin_amdgcn_s_barrier();
+        issue(s + RT_STAGES);     // into the stage every consumer has just left
+      }
+    } else {
+      Half h0, h1;
+      __builtin_amdgcn_s_barrier();  // stage 0 is in
+      asm volatile("" ::: "memory");
+      read_half(h0, 0, 0);
+      for (int s = 0; s < nsteps; ++s) {
+        chain_and_read(h0, h1, s, 1);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave no longer reads stage s
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // past the last stage this reads the stage the loaders refilled with the last
+        // step's data again; the values are never used
+        chain_and_read(h1, h0, s + 1, 0);
+      }
     }
-    // acc[4*b + r] of lane l: token th*16 + 4*(l/16) + r, expert e0 + eh*64 + 16*b + l%16
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int e = e0 + eh * 64 + 16 * b + l16;
+    if (loader) wait_vm<0>();       // nothing may land in a stage after this slab
+    __builtin_amdgcn_s_barrier();   // the stages may be refilled for the next slab
+    asm volatile("" ::: "memory");
+    if (!loader) {
+      // acc[r] of lane l: token 8*(r/4) + 4*(l/32) + r%4, expert e0 + 32*w + l%32
+      const int e = e0 + (wave & 3) * 32 + r32;
       const float bv = (bias != nullptr && e < E) ? as_global(bias)[e] : 0.0f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = acc[4 * b + r];
+      for (int r = 0; r < 16; ++r) {
+        float v = acc[r];
         if (bias != nullptr) v = __fadd_rn(v, bv);
-        if (e < MAX_EXPERTS) keys[(th * 16 + 4 * lq + r) * MAX_EXPERTS + e] = ordered_bits(v, e < E);
+        if (e < MAX_EXPERTS)
+          keys[(8 * (r >> 2) + 4 * kh + (r & 3)) * MAX_EXPERTS + e] = ordered_bits(v, e < E);
       }
     }
   }
   __syncthreads();
+#ifdef FMOE_DBG_STALL
+  const unsigned long long rt_c1 = stall_clock();
+  if (threadIdx.x == 0) {
+    sh_stall[0] = static_cast<unsigned>(rt_c1 - rt_c0);  // chain phase, cycles (packed >> 4 below)
+    sh_stall[1] = 0;
+    sh_stall[2] = 0;
+  }
+#endif
   // selection: the tokens are dealt out over all waves
   double* lex = sel + wave * MAX_TOPK;
   for (int i = 0; i < RT_TOK / WAVES; ++i) {
@@ -226,7 +354,9 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
         const int e = lane + 64 * j;
         val[j] = e < E ? keys[tl * MAX_EXPERTS + e] : 0u;
       }
+#ifndef FMOE_DBG_NO_SELECT  // timing experiment
       router_select_max(p, t, val, lex);
+#endif
     }
   }
 }
@@ -327,41 +457,6 @@ struct TileRows {
   unsigned toff[LQ];           // same for the token stage
 };
 
-#define FMOE_G1 __attribute__((address_space(1)))
-#define FMOE_L3 __attribute__((address_space(3)))
-
-__device__ __forceinline__ f32x16 mma32(const uint4& a, const uint4& b, f32x16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-
-// wait until at most N of this wave's vector-memory operations are outstanding
-// (they complete in order); nothing else is waited for
-template <int N>
-__device__ __forceinline__ void wait_vm() {
-  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
-
-// One wave-wide 16-byte-per-lane load from global memory straight into LDS:
-// lane l's 16 bytes from base + off land at LDS byte address lds_addr + 16*l.
-// Written as assembly so that the compiler does not order LDS reads of other
-// stages behind it; completion is tracked by hand with wait_vm.
-__device__ __forceinline__ void load_to_lds(unsigned off, const unsigned char* base, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :
-               : "v"(off), "s"(base), "s"(lds_addr)
-               : "memory");
-}
-
-#ifdef FMOE_DBG_STALL  // timing experiment: cycles a wave spends in the load wait and in the barrier
-__device__ unsigned long long g_stall[4];
-__shared__ unsigned sh_stall[4];  // last tile loop of wave 0: load wait, barrier, whole loop (cycles)
-__device__ __forceinline__ unsigned long long stall_clock() {
-  const unsigned long long t = __builtin_amdgcn_s_memtime();
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  return t;
-}
-#endif
 
 struct Frags {
   uint4 a[4];   // weight blocks
