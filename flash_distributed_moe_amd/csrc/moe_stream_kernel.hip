@@ -508,6 +508,16 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
                               : static_cast<size_t>(tile.row0 + row);
     bp[r] = reinterpret_cast<const elem*>(p.h) + hrow * p.I + g * EPV;
   }
+  // gate weight and destination of this lane's rows: fetched now, so that their
+  // latency is spent under the weight stream and not in the epilogue
+  float roww[RB];
+  int dstrow[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    const int row = min(r * 16 + r16, tile.rows - 1);
+    roww[r] = ldc(&p.row_w[tile.row0 + row]);
+    dstrow[r] = ldc(&p.perm[tile.row0 + row]);
+  }
   f32x4 acc[NA][RB];
 #pragma unroll
   for (int i = 0; i < NA; ++i)
@@ -523,8 +533,8 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
   for (int r = 0; r < RB; ++r) {
     const int row = r * 16 + r16;
     if (row < tile.rows) {
-      const float w = ldc(&p.row_w[tile.row0 + row]);
-      const size_t dst = static_cast<size_t>(ldc(&p.perm[tile.row0 + row])) * p.H;
+      const float w = roww[r];
+      const size_t dst = static_cast<size_t>(dstrow[r]) * p.H;
 #pragma unroll
       for (int b = 0; b < NA; ++b) {
         stc16(p.y + dst + n0 + 16 * b + 4 * g,
@@ -545,13 +555,26 @@ __device__ void combine_task(const Params& p, int t, int chunk) {
   const int c = chunk * COMBINE_COLS + lane * 4;
   if (c < p.H) {
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int k = 0; k < p.K; ++k) {
-      if (ldc(&p.topk_idx[static_cast<size_t>(t) * p.K + k]) < 0) continue;
-      const uint4 v = ldc16(p.y + (static_cast<size_t>(t) * p.K + k) * p.H + c);
-      s.x += __uint_as_float(v.x);
-      s.y += __uint_as_float(v.y);
-      s.z += __uint_as_float(v.z);
-      s.w += __uint_as_float(v.w);
+    // eight slots at a time: their validity and their rows are loaded together
+    // (one memory latency per group instead of two per slot), then added in slot order
+    for (int k0 = 0; k0 < p.K; k0 += 8) {
+      int idx[8];
+      uint4 v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int kk = min(k0 + k, p.K - 1);
+        idx[k] = ldc(&p.topk_idx[static_cast<size_t>(t) * p.K + kk]);
+        v[k] = ldc16(p.y + (static_cast<size_t>(t) * p.K + kk) * p.H + c);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        if (k0 + k < p.K && idx[k] >= 0) {
+          s.x += __uint_as_float(v[k].x);
+          s.y += __uint_as_float(v[k].y);
+          s.z += __uint_as_float(v[k].z);
+          s.w += __uint_as_float(v[k].w);
+        }
+      }
     }
     const size_t off = static_cast<size_t>(t) * p.H + c;
     if constexpr (DT::EPV == 8) {
@@ -777,6 +800,11 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
             ok = down_task<DT, 4, true>(p, tile, nblk, dep, nt1);
           }
         } else {
+          // the task reads its rows' gate weights and destinations up front
+          if (!perm_ready) {
+            if (!wait_flag(p, FLAG_PERM, lds_flag, lds_poller)) break;
+            perm_ready = true;
+          }
           unsigned* dep = &p.g1_done[aux].v;
           if (tile.rows <= 16) {
             ok = down_task<DT, 1, false>(p, tile, nblk, dep, nt1);

@@ -553,7 +553,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
 #endif
   auto step = [&](int ks, auto pending_tag, auto refill_tag, auto last_tag) {
     constexpr int PENDING = decltype(pending_tag)::value;
-    constexpr bool REFILL = decltype(refill_tag)::value;
+    constexpr int REFILL = decltype(refill_tag)::value;  // 1: refill with stage ks+STAGES
     constexpr bool LAST = decltype(last_tag)::value;
 #ifndef FMOE_DBG_NO_READS
     read(f1, ks, 1);
@@ -585,10 +585,11 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
         mfma_block(f1, g);
         __builtin_amdgcn_sched_barrier(0);
 #ifndef FMOE_DBG_NO_REFILL  // timing experiment: the main loop issues no loads
-        if (REFILL) {
+        if (REFILL == 1) {
           issue_one(ks + STAGES, 2 * g);
           issue_one(ks + STAGES, 2 * g + 1);
         }
+
 #endif
 #ifndef FMOE_DBG_NO_READS  // timing experiment: the main loop reads no fragments
 #pragma unroll
@@ -606,6 +607,8 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   using I8 = std::integral_constant<int, 2 * LQ>;   // one later stage in flight
   using I16 = std::integral_constant<int, 4 * LQ>;  // two later stages in flight
 
+  using R0 = std::integral_constant<int, 0>;
+  using R1 = std::integral_constant<int, 1>;
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) issue(s);  // ksteps >= STAGES for every admitted shape
   wait_vm<6 * LQ>();
@@ -613,11 +616,11 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   asm volatile("" ::: "memory");
   read(f0, 0, 0);
   int ks = 0;
-  for (; ks + STAGES < ksteps; ++ks) step(ks, I16{}, std::true_type{}, std::false_type{});
-  step(ks++, I16{}, std::false_type{}, std::false_type{});
-  step(ks++, I8{}, std::false_type{}, std::false_type{});
-  step(ks++, I0{}, std::false_type{}, std::false_type{});
-  step(ks, I0{}, std::false_type{}, std::true_type{});
+  for (; ks + STAGES < ksteps; ++ks) step(ks, I16{}, R1{}, std::false_type{});
+  step(ks++, I16{}, R0{}, std::false_type{});
+  step(ks++, I8{}, R0{}, std::false_type{});
+  step(ks++, I0{}, R0{}, std::false_type{});
+  step(ks, I0{}, R0{}, std::true_type{});
 #ifdef FMOE_DBG_STALL
   if (threadIdx.x == 0) {
     sh_stall[0] = static_cast<unsigned>(stall_vm);
