@@ -302,6 +302,111 @@ __device__ __noinline__ void scan_task(const Params& p) {
   }
 }
 
+// Small batches (every mask word, its prefix and every expert's offset fit the
+// wave's LDS slice): the same wave also writes the permutation, looking the
+// per-expert data up in LDS, so the whole stage costs two trips to memory — the
+// loads of masks and routing at the start, the stores at the end.
+constexpr int SCAN_LDS_WORDS = 1024;
+static_assert(SCAN_LDS_WORDS * 12 + MAX_EXPERTS * 4 <= ROUTER_LDS_FLOATS * 4, "scan tables exceed the wave's LDS");
+
+__device__ __noinline__ void scan_scatter_small_task(const Params& p) {
+  const RouteTables r = route_tables(p);
+  Control* ctl = p.ctl;
+  const int lane = lane_id();
+  const int epl = (r.E + 63) >> 6;
+  const int wact = (r.T + 63) >> 6;
+  const int n = r.T * r.K;
+  unsigned long long* lmask = reinterpret_cast<unsigned long long*>(lds_dyn + (threadIdx.x >> 6) * ROUTER_LDS_FLOATS);
+  int* lpre = reinterpret_cast<int*>(lmask + SCAN_LDS_WORDS);
+  int* loff = lpre + SCAN_LDS_WORDS;
+  constexpr int B = 8;  // routing entries per lane in flight together
+  // first round of routing entries: independent of the masks, fetched alongside them
+  int ee[B];
+  float ww[B];
+#pragma unroll
+  for (int b = 0; b < B; ++b) {
+    const int i = lane + 64 * b;
+    ee[b] = i < n ? ldc(&r.topk_idx[i]) : -1;
+    ww[b] = i < n ? ldc(&r.topk_w[i]) : 0.0f;
+  }
+  int base = 0, tile_base = 0;
+  for (int j = 0; j < epl; ++j) {
+    const int e = lane + 64 * j;
+    int c = 0;
+    if (e < r.E) {
+      const unsigned long long* m = r.masks + static_cast<size_t>(e) * r.W;
+      int* wp = r.word_prefix + static_cast<size_t>(e) * r.W;
+      for (int w0 = 0; w0 < wact; w0 += 4) {
+        unsigned long long mv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) mv[q] = w0 + q < wact ? ldc(&m[w0 + q]) : 0ull;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (w0 + q < wact) {
+            stc(&wp[w0 + q], c);
+            lmask[e * wact + w0 + q] = mv[q];
+            lpre[e * wact + w0 + q] = c;
+            c += __popcll(mv[q]);
+          }
+        }
+      }
+    }
+    const int incl = wave_inclusive_scan(c);
+    const int off = base + incl - c;
+    const int nt = (c + SKINNY_MT - 1) / SKINNY_MT;
+    const int tincl = wave_inclusive_scan(nt);
+    const int toff = tile_base + tincl - nt;
+    if (e < r.E) {
+      loff[e] = off;
+      stc(&r.expert_count[e], c);
+      stc(&r.expert_offset[e], off);
+      for (int i = 0; i < nt; ++i) {
+        if (toff + i < r.max_mtiles) {
+          stc16(&r.mtiles[toff + i],
+                make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + i * SKINNY_MT),
+                           static_cast<unsigned>(min(SKINNY_MT, c - i * SKINNY_MT)), 0u));
+        }
+      }
+    }
+    base += __shfl(incl, 63, 64);
+    tile_base += __shfl(tincl, 63, 64);
+  }
+  if (lane == 0) {
+    stc(&r.expert_offset[r.E], base);
+    if (tile_base > r.max_mtiles) {
+      or_relaxed(&ctl->error.v, ERR_CAPACITY);
+      tile_base = 0;
+    }
+    stc(&ctl->n_mtiles.v, static_cast<unsigned>(tile_base));
+  }
+  lds_wave_sync();
+  for (int i0 = lane; i0 < n; i0 += 64 * B) {
+    if (i0 != lane) {
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int i = i0 + 64 * b;
+        ee[b] = i < n ? ldc(&r.topk_idx[i]) : -1;
+        ww[b] = i < n ? ldc(&r.topk_w[i]) : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      if (ee[b] >= 0) {
+        const int i = i0 + 64 * b;
+        const int t = i / r.K;
+        const int wi = ee[b] * wact + (t >> 6);
+        const int pos = loff[ee[b]] + lpre[wi] + __popcll(lmask[wi] & ((1ull << (t & 63)) - 1ull));
+        stc(&r.perm[pos], i);
+        stc(&r.row_w[pos], ww[b]);
+      }
+    }
+  }
+  fence_release();
+  broadcast_flag(p, FLAG_SCAN);
+  broadcast_flag(p, FLAG_PERM);
+  lds_wave_sync();
+}
+
 __device__ void scatter_task(const Params& p, int t) {
   const RouteTables r = route_tables(p);
   const int lane = lane_id();
@@ -703,7 +808,11 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
       kind = 1;
       if (!wave_wait_ge(&ctl->router_done.v, T, ctl, p.spin_limit)) break;
       if (p.trace) t_ready = wall_clock64();
-      scan_task(p);
+      if (p.fuse_scatter && p.E * ((p.T + 63) >> 6) <= SCAN_LDS_WORDS) {
+        scan_scatter_small_task(p);
+      } else {
+        scan_task(p);
+      }
     } else if (tk < t_dense0) {
       kind = 2;
       aux = tk - t_scatter0;
