@@ -1,0 +1,121 @@
+"""Behaviour at the launcher boundary on the GPU: empty and oversized batches,
+the Python surface's checks, non-finite inputs, and the device-side time-out path
+(forced from the host with a tiny wait limit; the kernel still exits normally)."""
+import numpy as np
+import pytest
+import torch
+
+from flash_distributed_moe_amd import synth
+from oracle import oracle
+from tests.helpers import max_rel_err
+from tests.moe_case import GpuCase
+
+pytestmark = pytest.mark.gpu
+
+HIP_ERROR_UNKNOWN = 999
+
+
+def test_empty_batch_is_a_no_op():
+    cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=8, name="empty")
+    case = GpuCase(cfg)
+    try:
+        x = case.inp["tokens"][:0]
+        out = torch.empty_like(x)
+        case.launcher.launch(x, out)
+        torch.cuda.synchronize()
+        assert case.launcher.status()[0] == 0
+        # and the launcher still works afterwards
+        got = case.run()
+        case.check_outputs(case.inp["tokens"], got)
+    finally:
+        case.close()
+
+
+def test_more_tokens_than_max_tokens_is_refused(capfd):
+    cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=8, name="oversized")
+    case = GpuCase(cfg)
+    try:
+        big = torch.cat([case.inp["tokens"], case.inp["tokens"]], 0)
+        with pytest.raises(RuntimeError, match="hipError_t %d" % HIP_ERROR_UNKNOWN):
+            case.launcher.launch(big, torch.empty_like(big))
+        assert "exceeds max_tokens" in capfd.readouterr().out
+    finally:
+        case.close()
+
+
+def test_python_surface_checks():
+    cfg = synth.CONFIGS["tiny_f32"]
+    case = GpuCase(cfg)
+    try:
+        x = case.inp["tokens"]
+        with pytest.raises(RuntimeError, match="must be contiguous"):
+            case.launcher.launch(x.t().contiguous().t(), torch.empty_like(x))
+        with pytest.raises(RuntimeError, match="output shape must equal tokens shape"):
+            case.launcher.launch(x, torch.empty_like(x[:-1]))
+        with pytest.raises(RuntimeError, match="must be float32 or bfloat16"):
+            case.launcher.launch(x.to(torch.bfloat16), torch.empty_like(x, dtype=torch.bfloat16))
+        with pytest.raises(RuntimeError, match="CUDA tensor"):
+            case.launcher.launch(x.cpu(), torch.empty_like(x.cpu()))
+        assert case.launcher.valid
+        case.launcher.destroy()
+        assert not case.launcher.valid
+        with pytest.raises(RuntimeError, match="Launcher was destroyed"):
+            case.launcher.launch(x, torch.empty_like(x))
+    finally:
+        case.close()
+
+
+@pytest.mark.parametrize("name", ["tiny_f32", "qwen3_30b_decode"])
+def test_nan_and_all_equal_logits(name):
+    """A token row of NaNs selects nothing (every slot -1, output row 0), a row of
+    zeros makes every logit equal and must pick experts 0..k-1 in that order
+    (refTopk.h:36-58: strict '>' keeps the first of equals)."""
+    cfg = synth.CONFIGS[name].replace(T=6, name="nonfinite")
+    case = GpuCase(cfg)
+    try:
+        x = case.inp["tokens"].clone()
+        x[1] = float("nan")
+        x[4] = 0.0
+        out = torch.empty_like(x)
+        case.launcher.launch(x, out)
+        torch.cuda.synchronize()
+        assert case.launcher.status()[0] == 0
+        r = case.launcher.routing(cfg.T)
+        assert (r["topk_idx"][1] == -1).all()
+        assert list(r["topk_idx"][4]) == list(range(cfg.k))
+        case.check_routing(x, r)
+        got = out.float().cpu().numpy()
+        assert (got[1] == 0).all() and (got[4] == 0).all()
+        keep = [0, 2, 3, 5]
+        hw = case.host_weights()
+        ref, _, _ = oracle.forward(x.float().cpu().numpy()[keep], hw["gate"], hw["ffn1"], hw["ffn2"],
+                                   cfg.k)
+        tol = 1e-2 if cfg.dtype == "bf16" else 2e-5
+        assert max_rel_err(got[keep], ref) <= tol
+    finally:
+        case.close()
+
+
+@pytest.mark.parametrize("name,T,sched", [("qwen3_30b_decode", 64, 0), ("qwen3_30b_decode", 512, 2)])
+def test_device_wait_limit_is_reported_and_cleared(name, T, sched):
+    """With a wait limit of 100 ns every dependency wait that has to wait at all
+    gives up: the kernel ends normally, flashMoeStatus reports bit 1 and re-arms
+    the launcher, and the next launch with the normal limit is correct again."""
+    cfg = synth.CONFIGS[name].replace(T=T, name="timeout")
+    case = GpuCase(cfg, sched=sched)
+    try:
+        x = case.inp["tokens"]
+        good = case.run().clone()
+        case.launcher.set_wait_limit_ms(1e-4)
+        out = torch.empty_like(x)
+        case.launcher.launch(x, out)
+        torch.cuda.synchronize()
+        err, _ = case.launcher.status()
+        assert err & 1, "the shortened wait did not time out"
+        assert case.launcher.status()[0] == 0, "status must clear the error"
+        case.launcher.set_wait_limit_ms(2000.0)
+        again = case.run()
+        assert torch.equal(again, good)
+        case.check_outputs(x, again)
+    finally:
+        case.close()
