@@ -275,77 +275,6 @@ __device__ __forceinline__ void lds_wave_sync() {
   __builtin_amdgcn_wave_barrier();
 }
 
-// LDS scratch one wave needs for router_select
-constexpr int SELECT_LDS_BYTES = (MAX_EXPERTS + 2 * MAX_TOPK) * 8;
-
-// key[j] belongs to expert lane + 64*j; lk is LDS scratch private to the wave
-// (SELECT_LDS_BYTES). Writes the token's routing. Keys are
-// distinct (the index is part of the key), so a key's rank — how many keys are
-// greater — is its slot; ranks come from one pass over all keys in LDS.
-__device__ __forceinline__ void router_select(const Params& p, int t,
-                                              unsigned long long (&key)[MAX_EXPERTS / 64],
-                                              unsigned long long* lk) {
-  constexpr int MAXEPL = MAX_EXPERTS / 64;
-  const int lane = lane_id();
-  const int E = p.E, K = p.K;
-  unsigned long long* win = lk + MAX_EXPERTS;              // [MAX_TOPK] winning keys by slot
-  double* lex = reinterpret_cast<double*>(win + MAX_TOPK);  // [MAX_TOPK] exp terms
-  const int epl = (E + 63) >> 6;
-#pragma unroll
-  for (int j = 0; j < MAXEPL; ++j)
-    if (j < epl) lk[lane + 64 * j] = key[j];
-  if (lane < MAX_TOPK) win[lane] = 0ull;
-  lds_wave_sync();
-  int rank[MAXEPL];
-#pragma unroll
-  for (int j = 0; j < MAXEPL; ++j) rank[j] = 0;
-  const int n = epl * 64;
-  for (int i = 0; i < n; i += 2) {
-    const ulonglong2 o = *reinterpret_cast<const ulonglong2*>(lk + i);
-#pragma unroll
-    for (int j = 0; j < MAXEPL; ++j) rank[j] += (o.x > key[j] ? 1 : 0) + (o.y > key[j] ? 1 : 0);
-  }
-#pragma unroll
-  for (int j = 0; j < MAXEPL; ++j)
-    if (j < epl && key[j] != 0ull && rank[j] < K) win[rank[j]] = key[j];
-  lds_wave_sync();
-
-  int my_idx = -1;
-  float my_val = -FLT_MAX;
-  if (lane < K) {
-    const unsigned long long k64 = win[lane];
-    if (k64 != 0ull) {
-      my_idx = static_cast<int>(0xFFFFFFFFu - static_cast<unsigned>(k64 & 0xFFFFFFFFull));
-      unsigned u = static_cast<unsigned>(k64 >> 32);
-      u = (u & 0x80000000u) ? (u & 0x7FFFFFFFu) : ~u;
-      my_val = __uint_as_float(u);
-    }
-  }
-  // softmax over the K winners (descending, so the first is the maximum)
-  const unsigned long long k0 = win[0];
-  float v0f = -FLT_MAX;
-  if (k0 != 0ull) {
-    unsigned u = static_cast<unsigned>(k0 >> 32);
-    u = (u & 0x80000000u) ? (u & 0x7FFFFFFFu) : ~u;
-    v0f = __uint_as_float(u);
-  }
-  const double ex = lane < K ? exp(static_cast<double>(my_val) - static_cast<double>(v0f)) : 0.0;
-  if (lane < K) lex[lane] = ex;
-  lds_wave_sync();
-  double sum = 0.0;
-  for (int s = 0; s < K; ++s) sum += lex[s];
-  if (lane < K) {
-    const float w = sum <= 0.0 ? static_cast<float>(1.0 / static_cast<double>(K))
-                               : static_cast<float>(ex / sum);
-    stc(&p.topk_idx[static_cast<size_t>(t) * K + lane], my_idx);
-    stc(&p.topk_w[static_cast<size_t>(t) * K + lane], w);
-    if (my_idx >= 0) {
-      or_relaxed(&p.masks[static_cast<size_t>(my_idx) * p.W + (t >> 6)], 1ull << (t & 63));
-    }
-  }
-  lds_wave_sync();
-}
-
 // Order-preserving image of a logit: greater float <=> greater unsigned. Values
 // the reference's strict '>' against lowest() never admits (NaN, -inf,
 // -FLT_MAX) and experts out of range map to 0, which never wins.
@@ -373,8 +302,8 @@ __device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
   return a > b ? a : b;
 }
 
-// Same routing as router_select, by K rounds of "take the greatest logit that
-// is left, the lowest expert index among equals" (refTopk.h:36-58 keeps the
+// Top-k and gate weights of one token, by K rounds of "take the greatest logit
+// that is left, the lowest expert index among equals" (refTopk.h:36-58 keeps the
 // first of equal values because it compares with a strict '>'). val[j] is
 // ordered_bits of expert lane + 64*j. lex: MAX_TOPK doubles of LDS private to
 // the wave.

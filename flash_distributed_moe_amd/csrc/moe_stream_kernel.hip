@@ -840,26 +840,6 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
       wave_arrive(&p.g1_done[aux].v);
     } else {
       if (!have_dyn) {
-#ifdef FMOE_WARM_WEIGHTS  // experiment: slows the router more than it helps gate/up
-        // While the router runs, this wave has nothing to do: pull the weights
-        // its first gate/up task will most likely need (tile i is expert i when
-        // every expert is active) through the memory-side cache. A wrong guess
-        // only warms another task's weights.
-        if (p.ffn1_packed != nullptr && !dense && tk - t_dyn0 < static_cast<unsigned>(p.E) * nt1) {
-          const size_t task_bytes = static_cast<size_t>(p.H) * (2 * G1_NB * 16) * sizeof(typename DT::elem);
-          const char* src = reinterpret_cast<const char*>(p.ffn1_packed) +
-                            static_cast<size_t>(tk - t_dyn0) * task_bytes + lane * 16;
-          unsigned x = 0;
-          for (size_t off = 0; off < task_bytes; off += 16 * 1024) {
-            uint4 v[16];
-#pragma unroll
-            for (int u = 0; u < 16; ++u) v[u] = ld16(src + off + u * 1024);
-#pragma unroll
-            for (int u = 0; u < 16; ++u) x ^= v[u].x ^ v[u].w;
-          }
-          if (x == 0x9E3779B9u && p.T < 0) stc(&ctl->launches.v, x);  // never: keeps the loads alive
-        }
-#endif
         if (!wait_flag(p, FLAG_SCAN, lds_flag, lds_poller)) break;
         const unsigned nm = ldc(&ctl->n_mtiles.v);
         n1 = dense ? 0u : nm * nt1;

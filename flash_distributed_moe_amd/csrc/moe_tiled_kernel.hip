@@ -2,23 +2,24 @@
 // batches where an expert sees hundreds of rows (prefill) and the layer is
 // bound by MFMA throughput, bf16 only.
 //
-// One workgroup of 4 waves per CU draws workgroup-wide task tickets from the
-// same kind of counter as the streaming variant; tasks depend only on tasks
-// with smaller tickets. Stages (ticket order):
-//   router   32 tokens x all experts: logits in the oracle's summation order on
-//            the vector ALUs (a 4x4 register tile of sequential chains per
-//            thread, operands staged transposed in LDS), then top-k / softmax
-//   scan     per-expert counts, offsets, 256-row tile table
+// One workgroup of 8 waves per CU (two per SIMD) draws workgroup-wide task
+// tickets from the same kind of counter as the streaming variant; tasks depend
+// only on tasks with smaller tickets. Stages (ticket order):
+//   router   32 tokens x all experts: logits in the oracle's summation order
+//            as a chain of f32 matrix instructions (four waves multiply, four
+//            waves load through LDS), then top-k / softmax
+//   scan     one wave per expert: counts and running prefixes of its mask
+//            words; then one short task: offsets and the 256-row tile table
 //   scatter  32 tokens: permuted row of every (token, slot)
-//   gate/up  (row tile, 128 h columns): 256x256x64 MFMA tile, gate and up
+//   gate/up  (row tile, 128 h columns): 256x256 MFMA tile, gate and up
 //            columns side by side so that SiLU(gate)*up happens in registers
-//   down     (row tile, 256 output columns): same tile, weighted rows to y
+//   down     (row tile, 256 output columns): same tile, weighted bf16 rows to y
 //   combine  8 tokens: out = sum over slots of y
-// GEMM tile: 256 token rows x 256 weight rows, K stepped by 64 through
-// double-buffered LDS (rows padded to 144 bytes so 8 consecutive rows hit
-// different banks); each wave owns 128x128 of it as 4x4 MFMA 32x32x16 blocks,
-// 256 accumulator registers. Weight rows are the MFMA "A" operand so that a
-// lane ends up with runs of 4 consecutive output columns of one token row.
+// GEMM tile: 256 token rows x 256 weight rows, K stepped by 32 through four LDS
+// stages that are filled straight from global memory; each wave owns 128
+// weight rows x 64 token rows of it as 4x2 MFMA 32x32x16 blocks, 128
+// accumulator registers. Weight rows are the MFMA "A" operand so that a lane
+// ends up with runs of 4 consecutive output columns of one token row.
 //
 // Replaces, for this regime, the reference's moeKernel
 // (src/hip/kernel/moeKernel.h:37-107) and its TILE_M=1 GEMV tiles
@@ -160,15 +161,6 @@ __device__ __forceinline__ void load_to_lds(unsigned off, const unsigned char* b
                : "memory");
 }
 
-#ifdef FMOE_DBG_STALL  // timing experiment: cycles a wave spends in the load wait and in the barrier
-__device__ unsigned long long g_stall[4];
-__shared__ unsigned sh_stall[4];  // last tile loop of wave 0: load wait, barrier, whole loop (cycles)
-__device__ __forceinline__ unsigned long long stall_clock() {
-  const unsigned long long t = __builtin_amdgcn_s_memtime();
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  return t;
-}
-#endif
 
 // --------------------------------------------------------------------- router
 // Logits as in test/singleGPU/cpp/moe/reference/refGemm.h:21-24: one chain per
@@ -208,9 +200,6 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
   const bool loader = wave >= 4;
   const int t0 = uni(blk) * RT_TOK;
   const int nsteps = H >> 6;
-#ifdef FMOE_DBG_STALL
-  const unsigned long long rt_c0 = stall_clock();
-#endif
 
   for (int e0 = 0; e0 < E; e0 += 128) {
     // loader: load ld = 6*w + i fills the 64 16-byte slots from slot 64*ld on. Loads
@@ -232,9 +221,6 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
       const int src = min(step, nsteps - 1);  // past the end: refill with the last step (never read)
       const unsigned st = lds_addr + (step & (RT_STAGES - 1)) * RT_STAGE_BYTES +
                           ((wave & 3) * RT_LOADS) * 1024;
-#ifdef FMOE_DBG_RT_NOLOAD  // timing experiment
-      if (step > 3) return;
-#endif
 #pragma unroll
       for (int i = 0; i < RT_LOADS; ++i) {
         const bool tok = (wave & 3) * RT_LOADS + i < RT_TOK_LOADS;
@@ -334,14 +320,6 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
     }
   }
   __syncthreads();
-#ifdef FMOE_DBG_STALL
-  const unsigned long long rt_c1 = stall_clock();
-  if (threadIdx.x == 0) {
-    sh_stall[0] = static_cast<unsigned>(rt_c1 - rt_c0);  // chain phase, cycles (packed >> 4 below)
-    sh_stall[1] = 0;
-    sh_stall[2] = 0;
-  }
-#endif
   // selection: the tokens are dealt out over all waves
   double* lex = sel + wave * MAX_TOPK;
   for (int i = 0; i < RT_TOK / WAVES; ++i) {
@@ -354,9 +332,7 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
         const int e = lane + 64 * j;
         val[j] = e < E ? keys[tl * MAX_EXPERTS + e] : 0u;
       }
-#ifndef FMOE_DBG_NO_SELECT  // timing experiment
       router_select_max(p, t, val, lex);
-#endif
     }
   }
 }
@@ -490,11 +466,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   // load q (0..LQ-1: weight rows, LQ..2*LQ-1: token rows) of this wave's loads
   // of k-step ks into stage ks % STAGES
   auto issue_one = [&](int ks, int q) {
-#ifdef FMOE_DBG_NO_GLOBAL  // timing experiment: keep re-reading the first k-steps (cache hits)
-    const int src = ks & 3;
-#else
     const int src = ks;
-#endif
     const unsigned st = lds_addr + (ks & (STAGES - 1)) * STAGE_BYTES + wave * (LQ * 1024);
     if (q < LQ) {
       load_to_lds(rows.woff[q], rows.wbase + static_cast<size_t>(src) * (TK * 2), st + q * 1024);
@@ -531,11 +503,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
     if (j < JMAX) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-#ifdef FMOE_DBG_NO_MFMA  // timing experiment: consume the fragments without the matrix core
-        acc[i][j][0] += __uint_as_float(f.a[i].x ^ f.b[j].y);
-#else
         acc[i][j] = mma32(f.a[i], f.b[j], acc[i][j]);
-#endif
       }
     }
   };
@@ -547,55 +515,32 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   // instructions. PENDING: loads of later stages that may still be in flight
   // when stage ks+1 has to be complete (2 * LQ per stage).
   Frags f0, f1;
-#ifdef FMOE_DBG_STALL
-  unsigned long long stall_vm = 0, stall_bar = 0;
-  const unsigned long long loop_c0 = stall_clock();
-#endif
   auto step = [&](int ks, auto pending_tag, auto refill_tag, auto last_tag) {
     constexpr int PENDING = decltype(pending_tag)::value;
     constexpr int REFILL = decltype(refill_tag)::value;  // 1: refill with stage ks+STAGES
     constexpr bool LAST = decltype(last_tag)::value;
-#ifndef FMOE_DBG_NO_READS
     read(f1, ks, 1);
-#else
-    if (ks == 0) read(f1, ks, 1);
-#endif
 #pragma unroll
     for (int j = 0; j < WJ; ++j) mfma_block(f0, j);
     interleave_reads_and_mfma();
     __builtin_amdgcn_sched_barrier(0);
     if (!LAST) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // nobody still reads stage ks after the barrier
-#ifdef FMOE_DBG_STALL
-      const unsigned long long c0 = stall_clock();
-#endif
       wait_vm<PENDING>();
-#ifdef FMOE_DBG_STALL
-      const unsigned long long c1 = stall_clock();
-#endif
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
-#ifdef FMOE_DBG_STALL
-      const unsigned long long c2 = stall_clock();
-      stall_vm += c1 - c0;
-      stall_bar += c2 - c1;
-#endif
 #pragma unroll
       for (int g = 0; g < WJ; ++g) {
         mfma_block(f1, g);
         __builtin_amdgcn_sched_barrier(0);
-#ifndef FMOE_DBG_NO_REFILL  // timing experiment: the main loop issues no loads
         if (REFILL == 1) {
           issue_one(ks + STAGES, 2 * g);
           issue_one(ks + STAGES, 2 * g + 1);
         }
 
-#endif
-#ifndef FMOE_DBG_NO_READS  // timing experiment: the main loop reads no fragments
 #pragma unroll
         for (int i = g * (4 / WJ); i < (g + 1) * (4 / WJ); ++i) read_a(f0, ks + 1, 0, i);
         read_b(f0, ks + 1, 0, g);
-#endif
         __builtin_amdgcn_sched_barrier(0);
       }
     } else {
@@ -621,19 +566,6 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   step(ks++, I8{}, R0{}, std::false_type{});
   step(ks++, I0{}, R0{}, std::false_type{});
   step(ks, I0{}, R0{}, std::true_type{});
-#ifdef FMOE_DBG_STALL
-  if (threadIdx.x == 0) {
-    sh_stall[0] = static_cast<unsigned>(stall_vm);
-    sh_stall[1] = static_cast<unsigned>(stall_bar);
-    sh_stall[2] = static_cast<unsigned>(stall_clock() - loop_c0);
-  }
-  if (lane == 0) {
-    atomicAdd(&g_stall[0], stall_vm);
-    atomicAdd(&g_stall[1], stall_bar);
-    atomicAdd(&g_stall[2], stall_clock() - loop_c0);
-    atomicAdd(&g_stall[3], 1ull);
-  }
-#endif
   __syncthreads();  // the stages are free for the epilogue
 }
 
@@ -926,11 +858,7 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
       st16(reinterpret_cast<char*>(r) + 16,
            u32x4{static_cast<unsigned>(t_fetch), static_cast<unsigned>(t_fetch >> 32),
                  static_cast<unsigned>(t_ready), static_cast<unsigned>(t_ready >> 32)});
-#ifdef FMOE_DBG_STALL
-      const unsigned x0 = (sh_stall[0] >> 4) | ((sh_stall[1] >> 4) << 16), x1 = sh_stall[2];
-#else
       const unsigned x0 = 0u, x1 = 0u;
-#endif
       st16(reinterpret_cast<char*>(r) + 32,
            u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), x0, x1});
     }
