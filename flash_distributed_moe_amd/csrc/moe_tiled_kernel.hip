@@ -417,15 +417,16 @@ __device__ void tiled_scatter_task(const Params& p, int blk) {
 // Operands go HBM/L2 -> LDS directly (global_load_lds_dwordx4: lane l's 16
 // bytes land at LDS base + 16*l, from any global address), four stages of 32
 // k deep, so no register staging, no LDS write instructions and almost no VALU
-// work in the loop: with one wave per SIMD every VALU or LDS instruction of a
-// wave delays its next MFMA (measured: 8 cycles between VALU instructions of one
-// wave, ~65 cycles between its ds_read_b128 with 4 waves per CU).
+// work in the loop. A wave issues in order: every LDS read (about 20 cycles)
+// and every direct-to-LDS load it issues delays its own next MFMA, which is
+// why two waves share a SIMD here: one multiplies while the other issues.
 //
 // LDS stage layout: rows of 64 bytes (32 bf16), unpadded, weight rows 0..255
 // then token rows 0..255. Row R keeps its four 16-byte chunks permuted: chunk C
 // sits at position C ^ ((R >> 2) & 3), so the 16 rows a quarter-wave reads
-// together (256 bytes, all 64 banks) fall in 16 different 16-byte bank groups. One wave-wide load fills
-// 16 rows; lane l loads the chunk that belongs at position l & 3 of row l >> 2.
+// together (256 bytes, all 64 banks) fall in 16 different 16-byte bank groups.
+// One wave-wide load fills 16 rows; lane l loads the chunk that belongs at
+// position l & 3 of row l >> 2.
 struct TileRows {
   const unsigned char* wbase;  // uniform: expert's weight matrix
   const unsigned char* tbase;  // uniform: tokens, or this tile's h rows
