@@ -698,6 +698,30 @@ __device__ void combine_task(const Params& p, int t, int chunk) {
   }
 }
 
+// The combine items slot, slot + n_workers, ... of one worker (a function of its
+// own so that the worker loop's registers are not shared with it).
+template <typename DT>
+__device__ __noinline__ void combine_items(const Params& p, unsigned slot, unsigned nc,
+                                           unsigned ncomb, unsigned worker, unsigned id0,
+                                           long long t_fetch) {
+  const int lane = lane_id();
+  for (unsigned q = slot; q < nc; q += static_cast<unsigned>(p.n_workers)) {
+    const long long t_item = p.trace ? wall_clock64() : 0;
+    combine_task<DT>(p, static_cast<int>(q / ncomb), static_cast<int>(q % ncomb));
+    const unsigned id = id0 + q;
+    if (p.trace && lane == 0 && id < p.trace_cap) {
+      const long long t_end = wall_clock64();
+      TraceRec* r = p.trace + id;
+      st16(r, u32x4{id, 5u, worker, q / ncomb});
+      st16(reinterpret_cast<char*>(r) + 16,
+           u32x4{static_cast<unsigned>(t_fetch), static_cast<unsigned>(t_fetch >> 32),
+                 static_cast<unsigned>(t_item), static_cast<unsigned>(t_item >> 32)});
+      st16(reinterpret_cast<char*>(r) + 32,
+           u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), 0u, 0u});
+    }
+  }
+}
+
 // Wave-uniform bounded wait for this workgroup's copy of a phase flag. Only one
 // wave of the workgroup polls HBM; the others watch a word in LDS that the
 // polling wave sets (1 = flag seen, 2 = failed).
@@ -774,7 +798,7 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
   const unsigned ncomb = static_cast<unsigned>((p.H + COMBINE_COLS - 1) / COMBINE_COLS);
   const unsigned worker = blockIdx.x * waves_per_group + wave_in_group;
   unsigned n1 = 0, n2 = 0, nc = 0;
-  bool have_dyn = false, perm_ready = false, g2_ready = false;
+  bool have_dyn = false, perm_ready = false;
 
   // The first ticket of every worker is fixed (wave w of every workgroup before
   // wave w+1 of any, so the first tasks spread over all CUs); the shared counter
@@ -906,17 +930,19 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
         if (!ok) break;
         const unsigned old = wave_arrive(&ctl->g2_done.v);
         if (old == n2 - 1u) broadcast_flag(p, FLAG_G2);
-      } else if (j < n1 + n2 + nc) {
-        kind = 5;
-        if (!g2_ready) {
-          if (n2 != 0u && !wait_flag(p, FLAG_G2, lds_flag, lds_poller)) break;
-          g2_ready = true;
-        }
-        if (p.trace) t_ready = wall_clock64();
-        const unsigned q = j - n1 - n2;
-        aux = q / ncomb;
-        combine_task<DT>(p, static_cast<int>(q / ncomb), static_cast<int>(q % ncomb));
       } else {
+        // Every gate/up and down ticket has been handed out. The combine items
+        // need no order among themselves, so they are not ticketed one by one (a
+        // counter hands out only about 90 million tickets a second, which is what
+        // short combine tasks ran at). This last ticket of the worker is its
+        // arrival number instead: it takes items slot, slot + n_workers, ..., so
+        // the workers that run out of down tasks first do the combining, and one
+        // without an item leaves at once instead of spinning beside waves that
+        // still run down tasks.
+        const unsigned slot = j - n1 - n2;
+        if (slot >= nc) break;
+        if (n2 != 0u && !wait_flag(p, FLAG_G2, lds_flag, lds_poller)) break;
+        combine_items<DT>(p, slot, nc, ncomb, worker, t_dyn0 + n1 + n2, t_fetch);
         break;
       }
     }
