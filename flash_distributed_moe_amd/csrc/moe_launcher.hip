@@ -12,6 +12,7 @@
 //    in a HIP graph
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <new>
@@ -175,6 +176,18 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   // it pays while one 16-row MFMA block holds the whole batch and costs more
   // than the hidden routing prologue beyond that.
   p.dense = (T <= 16 && l->dense_ok) ? 1 : 0;
+  // Early gate/up tasks wait inside the kernel for the routing, so every routing
+  // task must be among the tickets the workers start with: they go to the first
+  // workgroups, four dot tasks and four select/scan tasks each (half of the
+  // workgroups at most, to leave workers for the weights).
+  const int dot_tasks = ((T + fmoe::ROUTER_TOK - 1) / fmoe::ROUTER_TOK) *
+                        ((d.experts + fmoe::ROUTER_EXP - 1) / fmoe::ROUTER_EXP);
+  const int routing_groups = std::max((dot_tasks + 3) / 4, (T + 4) / 4);
+  p.early = (!p.dense && p.fuse_scatter && T <= fmoe::EARLY_MAX_TOKENS &&
+             d.experts <= fmoe::SCAN_LDS_WORDS && d.experts <= L.max_mtiles &&
+             routing_groups <= p.n_groups / 2)
+                ? 1
+                : 0;
   p.tpad = (T + 15) / 16 * 16;
   p.max_mtiles = L.max_mtiles;
   p.spin_limit = l->spin_limit;

@@ -28,6 +28,10 @@ constexpr int G1_NB = FMOE_G1_NB;  // 16-wide column blocks per gate/up wave tas
 constexpr int G2_NB = FMOE_G2_NB;  // 16-wide column blocks per down wave task
 // Output columns summed by one combine task.
 constexpr int COMBINE_COLS = 256;
+constexpr int ROUTER_TOK = 8;    // streaming variant: tokens per router dot task
+constexpr int ROUTER_EXP = 8;    // streaming variant: experts per router dot task
+constexpr int SCAN_LDS_WORDS = 1024;  // mask words (experts x 64-token words) the small-batch scan keeps in LDS
+constexpr int EARLY_MAX_TOKENS = 64;   // batches up to this size take their gate/up weights before the routing is known
 constexpr int MAX_EXPERTS = 256;  // experts are spread 64 per wave register slot
 constexpr int MAX_TOPK = 32;
 
@@ -56,7 +60,8 @@ struct Control {
 // Phase flags, one line per workgroup: the worker that completes a phase
 // writes every workgroup's copy, so waiting workers poll a line nobody else
 // touches instead of queueing on one address.
-enum : int { FLAG_SCAN = 0, FLAG_PERM = 1, FLAG_G2 = 2 };
+// FLAG_ROUTED (streaming variant, early mode): every token's top-k entries are final.
+enum : int { FLAG_SCAN = 0, FLAG_PERM = 1, FLAG_G2 = 2, FLAG_ROUTED = 3 };
 struct alignas(128) WgFlags {
   unsigned f[32];
 };
@@ -118,6 +123,8 @@ struct Params {
   int n_groups;                    // workgroups in the grid
   int fuse_scatter;                // 1: the scan task also writes the permutation
   int dense;                       // 1: gate/up runs for every (expert, token) pair (small batches)
+  int early;                       // 1: row tile e belongs to expert e (empty or not), so gate/up tasks are
+                                   //    handed out at launch and fetch their first weights under the routing
   int tpad;                        // dense mode: h rows reserved per expert
   TraceRec* trace;    // null unless tracing; indexed by ticket
   unsigned trace_cap;

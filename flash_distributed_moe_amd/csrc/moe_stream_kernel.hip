@@ -46,8 +46,6 @@ namespace fmoe {
 // (k ascending). Each chain ends as a 64-bit candidate key in HBM. A "select"
 // task per token waits for all of the token's expert groups and picks the
 // winners.
-constexpr int ROUTER_TOK = 8;    // tokens per dot task
-constexpr int ROUTER_EXP = 8;    // experts per dot task
 constexpr int ROUTER_KC = 256;   // k-chunk staged in LDS
 constexpr int ROUTER_LD = ROUTER_KC + 4;  // LDS row stride in floats (bank spread)
 constexpr int ROUTER_LDS_FLOATS = 2 * ROUTER_EXP * ROUTER_LD;  // per wave
@@ -203,7 +201,8 @@ __device__ __noinline__ void router_select_task(const Params& p, int t) {
   if (lane == 0) stc(&p.tok_arrive[t], 0u);
   router_select_max(p, t, val,
                     reinterpret_cast<double*>(lds_dyn + (threadIdx.x >> 6) * ROUTER_LDS_FLOATS));
-  wave_arrive(&p.ctl->router_done.v);
+  const unsigned old = wave_arrive(&p.ctl->router_done.v);
+  if (p.early && old == static_cast<unsigned>(p.T) - 1u) broadcast_flag(p, FLAG_ROUTED);
 }
 
 // ------------------------------------------------------------- scan / scatter
@@ -306,7 +305,6 @@ __device__ __noinline__ void scan_task(const Params& p) {
 // wave's LDS slice): the same wave also writes the permutation, looking the
 // per-expert data up in LDS, so the whole stage costs two trips to memory — the
 // loads of masks and routing at the start, the stores at the end.
-constexpr int SCAN_LDS_WORDS = 1024;
 static_assert(SCAN_LDS_WORDS * 12 + MAX_EXPERTS * 4 <= ROUTER_LDS_FLOATS * 4, "scan tables exceed the wave's LDS");
 
 __device__ __noinline__ void scan_scatter_small_task(const Params& p) {
@@ -353,7 +351,8 @@ __device__ __noinline__ void scan_scatter_small_task(const Params& p) {
     }
     const int incl = wave_inclusive_scan(c);
     const int off = base + incl - c;
-    const int nt = (c + SKINNY_MT - 1) / SKINNY_MT;
+    // early mode: expert e owns tile e, empty or not (c <= 64 there)
+    const int nt = p.early ? (e < r.E ? 1 : 0) : (c + SKINNY_MT - 1) / SKINNY_MT;
     const int tincl = wave_inclusive_scan(nt);
     const int toff = tile_base + tincl - nt;
     if (e < r.E) {
@@ -413,6 +412,51 @@ __device__ void scatter_task(const Params& p, int t) {
   if (lane < r.K) scatter_entry(r, t * r.K + lane);
   const unsigned old = wave_arrive(&p.ctl->perm_done.v);
   if (old == static_cast<unsigned>(r.T) - 1u) broadcast_flag(p, FLAG_PERM);
+}
+
+// Wave-uniform bounded wait for this workgroup's copy of a phase flag. Only one
+// wave of the workgroup polls HBM; the others watch a word in LDS that the
+// polling wave sets (1 = flag seen, 2 = failed).
+__device__ __forceinline__ bool wait_flag(const Params& p, int which, unsigned* lds_flag,
+                                          unsigned* lds_poller) {
+  int ok = 1;
+  if (lane_id() == 0) {
+    while (true) {
+      const unsigned f = __hip_atomic_load(&lds_flag[which], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (f != 0u) {
+        ok = f == 1u;
+        break;
+      }
+      if (__hip_atomic_exchange(&lds_poller[which], 1u, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_WORKGROUP) == 0u) {
+        // this wave polls for the workgroup
+        const unsigned* g = &p.wgflags[blockIdx.x].f[which];
+        const long long t0 = wall_clock64();
+        unsigned spins = 0;
+        unsigned res = 1u;
+        while (ld_relaxed(g) == 0u) {
+          if ((++spins & 31u) == 0u && ld_relaxed(&p.ctl->error.v) != 0u) {
+            res = 2u;
+            break;
+          }
+          if (wall_clock64() - t0 > p.spin_limit) {
+            or_relaxed(&p.ctl->error.v, ERR_TIMEOUT);
+            res = 2u;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(16);
+        }
+        __hip_atomic_store(&lds_flag[which], res, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        ok = res == 1u;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+  }
+  ok = __builtin_amdgcn_readfirstlane(ok);
+  fence_acquire();
+  return ok != 0;
 }
 
 // ------------------------------------------------- streaming 16x16 MFMA sweep
@@ -493,7 +537,10 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
 // loads of 16 bytes per lane.
 template <int NA, int RB>
 struct RoundSteps {
-  static constexpr int value = RB == 1 ? (NA <= 2 ? 16 : 8) : (RB == 2 ? (NA <= 2 ? 8 : 4) : 4);
+#ifndef FMOE_U1
+#define FMOE_U1 8
+#endif
+  static constexpr int value = RB == 1 ? (NA <= 2 ? 2 * FMOE_U1 : FMOE_U1) : (RB == 2 ? (NA <= 2 ? 8 : 4) : 4);
 };
 
 // -------------------------------------------------------------------- gate/up
@@ -501,8 +548,55 @@ struct RoundSteps {
 // refExpertFFN1.h:51-65 (two GEMMs against the [2I,H] expert matrix, then
 // SiLU(gate) * up), accumulated on MFMA in float.
 // DENSE: the tile is (expert, all tokens): row r is token r, h row = row0 + r.
-template <typename DT, int RB, bool DENSE>
-__device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile, int nblk) {
+// The row tile of expert e read off the top-k table alone: its rows are the
+// entries i = token*K + slot that name e, in ascending i (the order the
+// permutation gives them), and its first row is the number of entries that name
+// a lower expert. Lanes 0..15 (and their copies in the other lane groups) get
+// the entry of row min(lane & 15, rows - 1). For batches of at most 64 tokens.
+__device__ __forceinline__ void tile_from_topk(const Params& p, int e, int& row0, int& rows,
+                                               int& entry) {
+  const int lane = lane_id();
+  const int r16 = lane & 15;
+  const int n = p.T * p.K;
+  int cnt = 0, lt = 0, idx = 0;
+  constexpr int B = 8;  // entries per lane in flight together
+  for (int i0 = 0; i0 < n; i0 += 64 * B) {
+    int ee[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int i = i0 + 64 * b + lane;
+      ee[b] = i < n ? ldc(&p.topk_idx[i]) : -1;
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const unsigned long long m = __ballot(ee[b] == e);
+      lt += __popcll(__ballot(ee[b] >= 0 && ee[b] < e));
+      const int pc = __popcll(m);
+      if (r16 >= cnt && r16 < cnt + pc) {
+        unsigned long long mm = m;
+        for (int j = cnt; j < r16; ++j) mm &= mm - 1ull;
+        idx = i0 + 64 * b + static_cast<int>(__builtin_ctzll(mm));
+      }
+      cnt += pc;
+    }
+  }
+  row0 = lt;
+  rows = cnt;
+  entry = __shfl(idx, max(min(r16, cnt - 1), 0), 64);
+}
+
+// EARLY (small batches: every expert owns the row tile of its own index, empty
+// or not, so tile -> weights is known at launch): the task is taken before the
+// routing exists. It issues its first round of weight loads at once, then waits
+// until every token's top-k entries are final and reads its rows off that table
+// (the scan and the permutation are only needed by the down tasks), so one round
+// of HBM latency and transfer per worker, and the scan, are off the critical path.
+// Returns 0: done (or the tile is empty), 1: the wait failed, 2 (EARLY only):
+// the tile has more than 16*RB rows, nothing was written, and the caller runs
+// the task again from the tile table with more row blocks.
+template <typename DT, int RB, bool DENSE, bool EARLY>
+__device__ __forceinline__ int gateup_body(const Params& p, TileDesc& tile, int nblk,
+                                           unsigned* lds_flag, unsigned* lds_poller) {
   typedef typename DT::elem elem;
   constexpr int EPV = DT::EPV;
   constexpr int NA = 2 * G1_NB;
@@ -531,19 +625,41 @@ __device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile, 
     }
   }
   const elem* bp[RB];
+  auto token_rows = [&] {
 #pragma unroll
-  for (int r = 0; r < RB; ++r) {
-    const int row = min(r * 16 + r16, tile.rows - 1);
-    const int tok = DENSE ? row : ldc(&p.perm[tile.row0 + row]) / p.K;
-    bp[r] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(tok) * p.H + g * EPV;
-  }
+    for (int r = 0; r < RB; ++r) {
+      const int row = min(r * 16 + r16, tile.rows - 1);
+      const int tok = DENSE ? row : ldc(&p.perm[tile.row0 + row]) / p.K;
+      bp[r] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(tok) * p.H + g * EPV;
+    }
+  };
+  if (!EARLY) token_rows();
   f32x4 acc[NA][RB];
 #pragma unroll
   for (int i = 0; i < NA; ++i)
 #pragma unroll
     for (int r = 0; r < RB; ++r) acc[i][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  stream_mma<DT, NA, RB, U, false>(ap, bp, p.H / (4 * EPV), astep, acc, [] { return true; });
+  int status = 0;
+  const bool ran = stream_mma<DT, NA, RB, U, false>(ap, bp, p.H / (4 * EPV), astep, acc, [&] {
+    if (EARLY) {
+      static_assert(!EARLY || RB == 1, "tile_from_topk serves one block of 16 rows");
+      if (!wait_flag(p, FLAG_ROUTED, lds_flag, lds_poller)) {
+        status = 1;
+        return false;
+      }
+      int entry;
+      tile_from_topk(p, tile.expert, tile.row0, tile.rows, entry);
+      if (tile.rows == 0) return false;
+      if (tile.rows > 16 * RB) {
+        status = 2;
+        return false;
+      }
+      bp[0] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(entry / p.K) * p.H + g * EPV;
+    }
+    return true;
+  });
+  if (!ran) return status;
 
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
@@ -568,6 +684,21 @@ __device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile, 
       }
     }
   }
+  return 0;
+}
+
+template <typename DT, int RB, bool DENSE>
+__device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile_in, int nblk) {
+  TileDesc tile = tile_in;
+  gateup_body<DT, RB, DENSE, false>(p, tile, nblk, nullptr, nullptr);
+}
+
+// tile.expert is set on entry; the rest of the descriptor is filled in once the
+// routing is known
+template <typename DT>
+__device__ __noinline__ int gateup_early_task(const Params& p, TileDesc& tile, int nblk,
+                                              unsigned* lds_flag, unsigned* lds_poller) {
+  return gateup_body<DT, 1, false, true>(p, tile, nblk, lds_flag, lds_poller);
 }
 
 // ----------------------------------------------------------------------- down
@@ -722,51 +853,6 @@ __device__ __noinline__ void combine_items(const Params& p, unsigned slot, unsig
   }
 }
 
-// Wave-uniform bounded wait for this workgroup's copy of a phase flag. Only one
-// wave of the workgroup polls HBM; the others watch a word in LDS that the
-// polling wave sets (1 = flag seen, 2 = failed).
-__device__ __forceinline__ bool wait_flag(const Params& p, int which, unsigned* lds_flag,
-                                          unsigned* lds_poller) {
-  int ok = 1;
-  if (lane_id() == 0) {
-    while (true) {
-      const unsigned f = __hip_atomic_load(&lds_flag[which], __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_WORKGROUP);
-      if (f != 0u) {
-        ok = f == 1u;
-        break;
-      }
-      if (__hip_atomic_exchange(&lds_poller[which], 1u, __ATOMIC_RELAXED,
-                                __HIP_MEMORY_SCOPE_WORKGROUP) == 0u) {
-        // this wave polls for the workgroup
-        const unsigned* g = &p.wgflags[blockIdx.x].f[which];
-        const long long t0 = wall_clock64();
-        unsigned spins = 0;
-        unsigned res = 1u;
-        while (ld_relaxed(g) == 0u) {
-          if ((++spins & 31u) == 0u && ld_relaxed(&p.ctl->error.v) != 0u) {
-            res = 2u;
-            break;
-          }
-          if (wall_clock64() - t0 > p.spin_limit) {
-            or_relaxed(&p.ctl->error.v, ERR_TIMEOUT);
-            res = 2u;
-            break;
-          }
-          __builtin_amdgcn_s_sleep(16);
-        }
-        __hip_atomic_store(&lds_flag[which], res, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        ok = res == 1u;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(8);
-    }
-  }
-  ok = __builtin_amdgcn_readfirstlane(ok);
-  fence_acquire();
-  return ok != 0;
-}
-
 // ---------------------------------------------------------------- worker loop
 template <typename DT>
 __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
@@ -799,18 +885,48 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
   const unsigned worker = blockIdx.x * waves_per_group + wave_in_group;
   unsigned n1 = 0, n2 = 0, nc = 0;
   bool have_dyn = false, perm_ready = false;
+  if (p.early) {  // one row tile per expert: the task counts do not depend on the routing
+    n1 = static_cast<unsigned>(p.E) * nt1;
+    n2 = static_cast<unsigned>(p.E) * nt2;
+    nc = T * ncomb;
+    have_dyn = true;
+  }
 
   // The first ticket of every worker is fixed (wave w of every workgroup before
   // wave w+1 of any, so the first tasks spread over all CUs); the shared counter
   // hands out the tickets after those.
   const unsigned n_workers = static_cast<unsigned>(p.n_workers);
   bool first = true;
+  unsigned first_tk = static_cast<unsigned>(wave_in_group) * gridDim.x + blockIdx.x;
+  unsigned dyn_base = n_workers;  // tickets below this are handed out statically
+  if (p.early) {
+    // The other workers start streaming weights at once, and a routing task
+    // whose loads queue behind those in its CU's memory pipeline runs a third
+    // slower. So the routing tasks sit together on the first workgroups: dot
+    // tasks on waves 0..3 (one per SIMD), select and scan tasks on waves 4..7.
+    // Workers of those workgroups without a routing task take dynamic tickets.
+    const unsigned nr = max((n_dot + 3u) / 4u, (T + 4u) / 4u);
+    const unsigned rest = gridDim.x - nr;
+    dyn_base = n_router + 1u + 8u * rest;
+    if (blockIdx.x >= nr) {
+      first_tk = n_router + 1u + static_cast<unsigned>(wave_in_group) * rest + (blockIdx.x - nr);
+    } else {
+      const unsigned q = blockIdx.x * 4u + (static_cast<unsigned>(wave_in_group) & 3u);
+      if (wave_in_group < 4) {
+        first_tk = q;
+        first = q < n_dot;
+      } else {
+        first_tk = n_dot + q;  // q == T: the scan
+        first = q <= T;
+      }
+    }
+  }
 
   while (true) {
     const long long t_fetch = p.trace ? wall_clock64() : 0;
-    unsigned tk = static_cast<unsigned>(wave_in_group) * gridDim.x + blockIdx.x;
+    unsigned tk = first_tk;
     if (!first) {
-      if (lane == 0) tk = n_workers + add_relaxed(&ctl->ticket.v, 1u);
+      if (lane == 0) tk = dyn_base + add_relaxed(&ctl->ticket.v, 1u);
       tk = __builtin_amdgcn_readfirstlane(tk);
     }
     first = false;
@@ -872,7 +988,32 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
         have_dyn = true;
       }
       const unsigned j = tk - t_dyn0;
-      if (j < n1) {
+      if (j < n1 && p.early) {
+        kind = 3;
+        aux = j / nt1;  // tile = expert
+        if (p.trace) t_ready = wall_clock64();
+        const int nblk = static_cast<int>(j % nt1);
+        TileDesc tile;
+        tile.expert = static_cast<int>(aux);
+        tile.row0 = 0;
+        tile.rows = 0;
+        tile.pad = 0;
+        const int st = gateup_early_task<DT>(p, tile, nblk, lds_flag, lds_poller);
+        if (st == 1) break;
+        if (st == 2) {
+          if (!perm_ready) {
+            if (!wait_flag(p, FLAG_PERM, lds_flag, lds_poller)) break;
+            perm_ready = true;
+          }
+          tile = ld_tile(&p.mtiles[aux]);
+          if (tile.rows <= 32) {
+            gateup_task<DT, 2, false>(p, tile, nblk);
+          } else {
+            gateup_task<DT, 4, false>(p, tile, nblk);
+          }
+        }
+        wave_arrive(&p.g1_done[aux].v);
+      } else if (j < n1) {
         kind = 3;
         aux = j / nt1;
         if (!perm_ready) {
@@ -894,6 +1035,10 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
         kind = 4;
         aux = (j - n1) / nt2;
         const int nblk = static_cast<int>((j - n1) % nt2);
+        if (p.early && !perm_ready) {  // nothing has waited for the tile table yet
+          if (!wait_flag(p, FLAG_PERM, lds_flag, lds_poller)) break;
+          perm_ready = true;
+        }
         if (p.trace) t_ready = wall_clock64();
         const TileDesc tile = ld_tile(&p.mtiles[aux]);
         bool ok;
@@ -919,7 +1064,9 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
             perm_ready = true;
           }
           unsigned* dep = &p.g1_done[aux].v;
-          if (tile.rows <= 16) {
+          if (tile.rows == 0) {  // early mode keeps the tiles of unused experts
+            ok = true;
+          } else if (tile.rows <= 16) {
             ok = down_task<DT, 1, false>(p, tile, nblk, dep, nt1);
           } else if (tile.rows <= 32) {
             ok = down_task<DT, 2, false>(p, tile, nblk, dep, nt1);
@@ -974,6 +1121,7 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
       stc(&p.wgflags[g].f[FLAG_SCAN], 0u);
       stc(&p.wgflags[g].f[FLAG_PERM], 0u);
       stc(&p.wgflags[g].f[FLAG_G2], 0u);
+      stc(&p.wgflags[g].f[FLAG_ROUTED], 0u);
     }
     if (lane == 0) {
       stc(&ctl->launches.v, ldc(&ctl->launches.v) + 1u);
