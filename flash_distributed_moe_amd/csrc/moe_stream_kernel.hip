@@ -479,7 +479,7 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int i = 0; i < NA; ++i) a[u][i] = ld16(ap[i] + static_cast<size_t>(s + u) * astep);
+      for (int i = 0; i < NA; ++i) a[u][i] = ld16_once(ap[i] + static_cast<size_t>(s + u) * astep);
   };
   auto load_b = [&](int s) {
 #pragma unroll
@@ -522,7 +522,7 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
   for (; s < ksteps; ++s) {  // remainder when ksteps is not a multiple of U
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      const uint4 av = ld16(ap[i] + static_cast<size_t>(s) * astep);
+      const uint4 av = ld16_once(ap[i] + static_cast<size_t>(s) * astep);
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
         const typename DT::elem* q = bp[r] + static_cast<size_t>(s) * KS;
