@@ -760,7 +760,10 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
 #pragma unroll
     for (int r = 0; r < RB; ++r) acc[i][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const bool ok = stream_mma<DT, NA, RB, U, true>(ap, bp, p.I / (4 * EPV), astep, acc, [&] {
+  // The h rows are read with ordinary loads: their writers stored them through
+  // to device-coherent memory and released before bumping the counter, and the
+  // wait below ends with an agent-scope acquire, which drops any stale copy.
+  const bool ok = stream_mma<DT, NA, RB, U, false>(ap, bp, p.I / (4 * EPV), astep, acc, [&] {
     return wave_wait_ge(dep, dep_target, p.ctl, p.spin_limit);
   });
   if (!ok) return false;
