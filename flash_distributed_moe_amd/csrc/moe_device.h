@@ -85,7 +85,11 @@ __device__ __forceinline__ void stc16(void* p, const uint4& v) {
 __device__ __forceinline__ void st16_through(void* p, const uint4& v) {
   typedef unsigned v4u __attribute__((ext_vector_type(4)));
   const v4u d = {v.x, v.y, v.z, v.w};
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(d) : "memory");
+  // The two idle cycles after the store are the wait states the hardware needs
+  // before a vector instruction may overwrite the data registers of a store
+  // wider than 8 bytes; the compiler inserts them for its own stores, but does
+  // not look inside assembly.
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(d) : "memory");
 }
 __device__ __forceinline__ TileDesc ld_tile(const TileDesc* t) {
   const uint4 v = ldc16(t);

@@ -768,15 +768,17 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
   });
   if (!ok) return false;
 
+  float* const ybase = p.y + n0 + 4 * g;
+  const size_t ystride = static_cast<size_t>(p.H);
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
     const int row = r * 16 + r16;
     if (row < tile.rows) {
       const float w = roww[r];
-      const size_t dst = static_cast<size_t>(dstrow[r]) * p.H;
+      float* const yrow = ybase + static_cast<size_t>(dstrow[r]) * ystride;
 #pragma unroll
       for (int b = 0; b < NA; ++b) {
-        stc16(p.y + dst + n0 + 16 * b + 4 * g,
+        st16_through(yrow + 16 * b,
               make_uint4(__float_as_uint(acc[b][r][0] * w), __float_as_uint(acc[b][r][1] * w),
                          __float_as_uint(acc[b][r][2] * w), __float_as_uint(acc[b][r][3] * w)));
       }
@@ -803,7 +805,7 @@ __device__ void combine_task(const Params& p, int t, int chunk) {
       for (int k = 0; k < 8; ++k) {
         const int kk = min(k0 + k, p.K - 1);
         idx[k] = ldc(&p.topk_idx[static_cast<size_t>(t) * p.K + kk]);
-        v[k] = ldc16(p.y + (static_cast<size_t>(t) * p.K + kk) * p.H + c);
+        v[k] = ld16_once(p.y + (static_cast<size_t>(t) * p.K + kk) * p.H + c);
       }
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
