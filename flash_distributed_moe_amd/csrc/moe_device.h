@@ -176,6 +176,29 @@ __device__ __forceinline__ uint4 ld16(const void* p) {
   const u32x4 v = *as_global(reinterpret_cast<const u32x4*>(p));
   return make_uint4(v.x, v.y, v.z, v.w);
 }
+// a pointer that is the same in every lane, pinned to scalar registers
+template <typename T>
+__device__ __forceinline__ T* uniform_ptr(T* ptr) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
+  return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
+// 16 bytes read at agent scope (one instruction; an atomic load carries 8 at
+// most): the load bypasses whatever this XCD's L2 holds for the line, so it sees
+// what other XCDs have written through. `base` is uniform, `off` < `bytes`.
+struct CoherentBuffer {
+  __amdgpu_buffer_rsrc_t rsrc;
+};
+__device__ __forceinline__ CoherentBuffer coherent_buffer(const void* base, unsigned bytes) {
+  CoherentBuffer b;
+  b.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+  return b;
+}
+__device__ __forceinline__ uint4 ld16_agent(const CoherentBuffer& b, unsigned off) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(b.rsrc, static_cast<int>(off), 0, 16 /* sc1 */);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
 // 16 bytes that are used once (expert weights): marked non-temporal, so that
 // they do not push the token rows and the routing tables out of the L2
 __device__ __forceinline__ uint4 ld16_once(const void* p) {

@@ -29,6 +29,9 @@
 // (src/hip/kernel/tasks/*.h) and its queue (src/hip/taskSystem/*.h).
 #include "moe_device.h"
 
+#ifndef FMOE_COH_B
+#define FMOE_COH_B true
+#endif
 namespace fmoe {
 
 // --------------------------------------------------------------------- router
@@ -469,11 +472,22 @@ __device__ __forceinline__ bool wait_flag(const Params& p, int which, unsigned* 
 template <typename DT, int NA, int RB, int U, bool COH_B, typename Pre>
 __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[NA],
                                            const typename DT::elem* const (&bp)[RB], int ksteps,
-                                           int astep, f32x4 (&acc)[NA][RB], Pre pre) {
+                                           int astep, f32x4 (&acc)[NA][RB], Pre pre,
+                                           const void* bbase = nullptr, unsigned bbytes = 0) {
   // astep: elements between one k-step's A fragment and the next (4*EPV in the
   // caller's row-major layout, NA*64*EPV in the packed layout)
   constexpr int KS = 4 * DT::EPV;
   uint4 a[U][NA], b[U][RB];
+  // COH_B: the B rows (inside [bbase, bbase + bbytes)) were written by other
+  // workers during this launch and are read at agent scope
+  const CoherentBuffer cb = coherent_buffer(bbase, bbytes);
+  auto ld_b = [&](const typename DT::elem* q) {
+    if (COH_B) {
+      return ld16_agent(cb, static_cast<unsigned>(reinterpret_cast<const char*>(q) -
+                                                  reinterpret_cast<const char*>(bbase)));
+    }
+    return ld16(q);
+  };
 
   auto load_a = [&](int s) {
 #pragma unroll
@@ -487,7 +501,7 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
         const typename DT::elem* q = bp[r] + static_cast<size_t>(s + u) * KS;
-        b[u][r] = COH_B ? ldc16(q) : ld16(q);
+        b[u][r] = ld_b(q);
       }
   };
   auto mma = [&]() {
@@ -526,7 +540,7 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
         const typename DT::elem* q = bp[r] + static_cast<size_t>(s) * KS;
-        acc[i][r] = mma16<DT>(av, COH_B ? ldc16(q) : ld16(q), acc[i][r]);
+        acc[i][r] = mma16<DT>(av, ld_b(q), acc[i][r]);
       }
     }
   }
@@ -734,6 +748,11 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
     for (int b = 0; b < NA; ++b)
       ap[b] = w2 + static_cast<size_t>(n0 + 16 * b + r16) * p.I + g * EPV;
   }
+  // the part of h this tile reads (uniform; the offsets inside it fit 32 bits)
+  const size_t hrow0 = DENSE ? static_cast<size_t>(tile.expert) * p.tpad : static_cast<size_t>(tile.row0);
+  const elem* hbase = uniform_ptr(reinterpret_cast<const elem*>(p.h) + hrow0 * p.I);
+  const unsigned hbytes = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(
+      (DENSE ? p.tpad : tile.rows) * p.I * static_cast<int>(sizeof(elem))));
   const elem* bp[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
@@ -760,12 +779,12 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
 #pragma unroll
     for (int r = 0; r < RB; ++r) acc[i][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // The h rows are read with ordinary loads: their writers stored them through
-  // to device-coherent memory and released before bumping the counter, and the
-  // wait below ends with an agent-scope acquire, which drops any stale copy.
-  const bool ok = stream_mma<DT, NA, RB, U, false>(ap, bp, p.I / (4 * EPV), astep, acc, [&] {
+  // The h rows are read at agent scope: two gate/up tasks, possibly on different
+  // XCDs, each write half of a 128-byte line of h, so this XCD's L2 may hold a
+  // line one of its own tasks wrote before the other half existed.
+  const bool ok = stream_mma<DT, NA, RB, U, FMOE_COH_B>(ap, bp, p.I / (4 * EPV), astep, acc, [&] {
     return wave_wait_ge(dep, dep_target, p.ctl, p.spin_limit);
-  });
+  }, hbase, hbytes);
   if (!ok) return false;
 
   float* const ybase = p.y + n0 + 4 * g;
