@@ -72,6 +72,9 @@ def test_ragged_token_counts_bf16(T):
     (33, 256, 32, 1, 96, "bf16"),   # top-1
     (40, 192, 200, 6, 160, "bf16"),  # E not a multiple of 64
     (100, 64, 4, 2, 32, "bf16"),    # > 64 rows per expert: several row tiles
+    (64, 64, 4, 2, 32, "bf16"),     # small batch whose experts get ~32 rows: early tasks re-run with more row blocks
+    (48, 128, 2, 1, 64, "bf16"),    # ~24 rows per expert, top-1
+    (60, 128, 3, 3, 64, "f32"),     # k == E: 60 rows in every expert
 ])
 def test_odd_shapes(shape):
     T, H, E, k, I, dt = shape
