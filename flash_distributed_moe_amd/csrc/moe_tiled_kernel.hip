@@ -789,7 +789,7 @@ __device__ __noinline__ void tiled_combine_task(const Params& p, int blk) {
       uint4 v[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k)
-        if (k0 + k < K) v[k] = ld16(yrow + static_cast<size_t>(k0 + k) * H);
+        if (k0 + k < K) v[k] = ld16_once(yrow + static_cast<size_t>(k0 + k) * H);
 #pragma unroll
       for (int k = 0; k < 8; ++k)
         if (k0 + k < K && ((valid >> (k0 + k)) & 1u)) {
