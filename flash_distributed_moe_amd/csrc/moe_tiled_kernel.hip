@@ -454,10 +454,14 @@ __device__ __forceinline__ void interleave_reads_and_mfma() {
 // acc[i][j] (+)= W-block i (32 weight rows) x token-block j (32 token rows).
 // wblk[i]: first weight row of block i inside the weight stage; tokens of this
 // wave start at tok0. JMAX: token blocks of this wave that are computed.
-// Every wave loads its share of each stage whatever its JMAX.
-template <int JMAX>
+// Every wave loads its share of the weight rows of each stage whatever its
+// JMAX; TOKL: it also loads its 32 token rows (false when they all lie past the
+// tile's end: those stage rows then keep whatever they held, and feed only
+// output rows that the epilogue drops).
+template <int JMAX, bool TOKL>
 __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, const int (&wblk)[4],
                                             int tok0, f32x16 (&acc)[4][WJ]) {
+  constexpr int NLQ = TOKL ? 2 * LQ : LQ;  // this wave's loads per stage
   const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
   const int r32 = lane & 31, kq = lane >> 5;
   const unsigned char* lds = lds_raw;
@@ -478,7 +482,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   };
   auto issue = [&](int ks) {
 #pragma unroll
-    for (int q = 0; q < 2 * LQ; ++q) issue_one(ks, q);
+    for (int q = 0; q < NLQ; ++q) issue_one(ks, q);
   };
 
   // per-lane read offsets: row r32 of a block, chunk kk*2+kq at its permuted position
@@ -535,8 +539,8 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
         mfma_block(f1, g);
         __builtin_amdgcn_sched_barrier(0);
         if (REFILL == 1) {
-          issue_one(ks + STAGES, 2 * g);
-          issue_one(ks + STAGES, 2 * g + 1);
+          if (2 * g < NLQ) issue_one(ks + STAGES, 2 * g);
+          if (2 * g + 1 < NLQ) issue_one(ks + STAGES, 2 * g + 1);
         }
 
 #pragma unroll
@@ -550,14 +554,14 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
     }
   };
   using I0 = std::integral_constant<int, 0>;
-  using I8 = std::integral_constant<int, 2 * LQ>;   // one later stage in flight
-  using I16 = std::integral_constant<int, 4 * LQ>;  // two later stages in flight
+  using I8 = std::integral_constant<int, NLQ>;       // one later stage in flight
+  using I16 = std::integral_constant<int, 2 * NLQ>;  // two later stages in flight
 
   using R0 = std::integral_constant<int, 0>;
   using R1 = std::integral_constant<int, 1>;
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) issue(s);  // ksteps >= STAGES for every admitted shape
-  wait_vm<6 * LQ>();
+  wait_vm<3 * NLQ>();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   read(f0, 0, 0);
@@ -574,13 +578,23 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
 // Rounding it up is safe: rows past the tile's end are clamped copies whose
 // results the epilogue drops.
 __device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, const int (&wblk)[4],
-                                          int tok0, int jmax, f32x16 (&acc)[4][WJ]) {
-  if (jmax > WJ / 2) {
-    tile_gemm_j<WJ>(rows, ksteps, wblk, tok0, acc);
-  } else if (jmax > 0) {
-    tile_gemm_j<WJ / 2>(rows, ksteps, wblk, tok0, acc);
+                                          int tok0, int jmax, bool tokl, f32x16 (&acc)[4][WJ]) {
+  if (tokl) {
+    if (jmax > WJ / 2) {
+      tile_gemm_j<WJ, true>(rows, ksteps, wblk, tok0, acc);
+    } else if (jmax > 0) {
+      tile_gemm_j<WJ / 2, true>(rows, ksteps, wblk, tok0, acc);
+    } else {
+      tile_gemm_j<0, true>(rows, ksteps, wblk, tok0, acc);
+    }
   } else {
-    tile_gemm_j<0>(rows, ksteps, wblk, tok0, acc);
+    if (jmax > WJ / 2) {
+      tile_gemm_j<WJ, false>(rows, ksteps, wblk, tok0, acc);
+    } else if (jmax > 0) {
+      tile_gemm_j<WJ / 2, false>(rows, ksteps, wblk, tok0, acc);
+    } else {
+      tile_gemm_j<0, false>(rows, ksteps, wblk, tok0, acc);
+    }
   }
 }
 
@@ -621,6 +635,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
   const int wblk[4] = {wn * 64, wn * 64 + 32, G1_COLS + wn * 64, G1_COLS + wn * 64 + 32};
   const int tok0 = wm * (32 * WJ);
   const int jmax = uni(min(WJ, max(0, (tile.rows - tok0 + 31) / 32)));
+  const bool tokl = wave * (16 * LQ) < tile.rows;  // some of the token rows this wave loads exist
   unsigned short* h = uni(reinterpret_cast<unsigned short*>(p.h)) +
                       static_cast<size_t>(tile.row0) * I + n0 + wn * 64;
   f32x16 acc[4][WJ];
@@ -631,7 +646,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  tile_gemm(rows, H / TK, wblk, tok0, jmax, acc);
+  tile_gemm(rows, H / TK, wblk, tok0, jmax, tokl, acc);
 
   // Epilogue through LDS (the stage buffers are free now): each wave turns its
   // 32-token x 64-column blocks into full 128-byte row segments of h. Nothing
@@ -696,6 +711,7 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
   const int wblk[4] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
   const int tok0 = wm * (32 * WJ);
   const int jmax = uni(min(WJ, max(0, (tile.rows - tok0 + 31) / 32)));
+  const bool tokl = wave * (16 * LQ) < tile.rows;  // some of the token rows this wave loads exist
   const int r32 = lane & 31, kq = lane >> 5;
   // y rows are bf16 here: H values per (token, slot)
   unsigned short* y = uni(reinterpret_cast<unsigned short*>(p.y)) + n0 + wn * 128 + (lane & 15) * 8;
@@ -721,7 +737,7 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  tile_gemm(rows, I / TK, wblk, tok0, jmax, acc);
+  tile_gemm(rows, I / TK, wblk, tok0, jmax, tokl, acc);
 
   // Epilogue through LDS: 32-token x 128-column blocks become 256-byte row
   // segments of y (bf16), scaled by the row's gate weight, at the row's
