@@ -427,12 +427,23 @@ __device__ void tiled_scatter_task(const Params& p, int blk) {
 // together (256 bytes, all 64 banks) fall in 16 different 16-byte bank groups.
 // One wave-wide load fills 16 rows; lane l loads the chunk that belongs at
 // position l & 3 of row l >> 2.
+// Weights come either from the caller's row-major matrices (64 bytes of each of
+// 16 rows per load) or, when the launcher keeps the packed copy, from that: the
+// streaming variant's layout holds every 16-row block of a k-step as one
+// contiguous 1 KiB run [chunk 0..3][row 0..15][16 B], which a load fetches as
+// eight whole cache lines. Measured with these loads on all CUs and four
+// workgroups per XCD sharing a tile: 40 us per 2 MiB tile from 1 KiB runs, 50 us
+// from 64-byte row segments 4096 bytes apart (all hits: 20 against 35 us). The
+// block keeps that order in LDS; the fragment reads below allow for it.
 struct TileRows {
-  const unsigned char* wbase;  // uniform: expert's weight matrix
-  const unsigned char* tbase;  // uniform: tokens, or this tile's h rows
-  unsigned woff[LQ];           // byte offset of this lane's chunk of weight-stage row wave*16*LQ+q*16+(lane>>2)
-  unsigned toff[LQ];           // same for the token stage
+  const unsigned char* wbase[LQ];  // uniform: where this wave's weight load q starts at k-step 0
+  const unsigned char* tbase;      // uniform: tokens, or this tile's h rows
+  unsigned wkstride;               // uniform: bytes from one k-step's weights to the next
+  bool wpacked;                    // uniform: weight blocks are 1 KiB runs
+  unsigned woff[LQ];               // byte offset of this lane's 16 bytes of weight load q
+  unsigned toff[LQ];               // token stage: this lane's chunk of stage row wave*16*LQ+q*16+(lane>>2)
 };
+static_assert(G1_NB == 2 && G2_NB == 4, "the tiled variant reads the packed copy as 32+32-row and 64-row tasks");
 
 
 struct Frags {
@@ -474,7 +485,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
     const int src = ks;
     const unsigned st = lds_addr + (ks & (STAGES - 1)) * STAGE_BYTES + wave * (LQ * 1024);
     if (q < LQ) {
-      load_to_lds(rows.woff[q], rows.wbase + static_cast<size_t>(src) * (TK * 2), st + q * 1024);
+      load_to_lds(rows.woff[q], rows.wbase[q] + static_cast<size_t>(src) * rows.wkstride, st + q * 1024);
     } else {
       load_to_lds(rows.toff[q - LQ], rows.tbase + static_cast<size_t>(src) * (TK * 2),
                   st + TN * TK * 2 + (q - LQ) * 1024);
@@ -490,8 +501,12 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
   const int rd0 = r32 * 64 + ((kq ^ swz) << 4);        // kk = 0
   const int rd1 = r32 * 64 + (((kq ^ swz) ^ 2) << 4);  // kk = 1
 
+  // packed weight blocks: row r32 of a 32-row block is row r32 % 16 of its 16-row
+  // block r32 / 16, chunk C of it at ((C * 16) + row) * 16
+  const int ra0 = rows.wpacked ? (r32 >> 4) * 1024 + ((kq * 16 + (r32 & 15)) << 4) : rd0;
+  const int ra1 = rows.wpacked ? (r32 >> 4) * 1024 + (((2 + kq) * 16 + (r32 & 15)) << 4) : rd1;
   auto read_a = [&](Frags& f, int ks, int kk, int i) {
-    const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? rd0 : rd1);
+    const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? ra0 : ra1);
     if (JMAX > 0) f.a[i] = *reinterpret_cast<const uint4*>(st + wblk[i] * 64);
   };
   auto read_b = [&](Frags& f, int ks, int kk, int j) {
@@ -619,14 +634,27 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
   const unsigned short* w13 = uni(reinterpret_cast<const unsigned short*>(p.ffn1)) +
                               static_cast<size_t>(tile.expert) * 2 * I * H;
   TileRows rows;
-  rows.wbase = reinterpret_cast<const unsigned char*>(w13);
+  rows.wpacked = uni(p.ffn1_packed != nullptr ? 1 : 0) != 0;
+  rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
   rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
 #pragma unroll
   for (int q = 0; q < LQ; ++q) {
     const int row = stage_row(q);
-    // weight stage rows 0..127: gate rows n0+row, 128..255: up rows I+n0+(row-128)
-    const int wrow = row < G1_COLS ? n0 + row : I + n0 + (row - G1_COLS);
-    rows.woff[q] = static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+    if (rows.wpacked) {
+      // stage block B (16 rows): gate blocks 0..7, up blocks 8..15; the packed task
+      // of 32 h columns holds gate blocks 0,1 and up blocks 2,3 of every k-step
+      const int B = uni(static_cast<int>(threadIdx.x >> 6)) * LQ + q;
+      const int half = B >> 3, b8 = B & 7;
+      const size_t task = static_cast<size_t>(tile.expert) * (I / 32) + (n0 / 32 + (b8 >> 1));
+      rows.wbase[q] = uni(reinterpret_cast<const unsigned char*>(p.ffn1_packed)) +
+                      task * (static_cast<size_t>(H / 32) * 4096) + (2 * half + (b8 & 1)) * 1024;
+      rows.woff[q] = (threadIdx.x & 63) * 16;
+    } else {
+      // weight stage rows 0..127: gate rows n0+row, 128..255: up rows I+n0+(row-128)
+      const int wrow = row < G1_COLS ? n0 + row : I + n0 + (row - G1_COLS);
+      rows.wbase[q] = reinterpret_cast<const unsigned char*>(w13);
+      rows.woff[q] = static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+    }
     const int tok = ldc(&p.perm[tile.row0 + min(row, tile.rows - 1)]) / K;
     rows.toff[q] = static_cast<unsigned>(tok) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
   }
@@ -696,13 +724,24 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
   const unsigned short* w2 = uni(reinterpret_cast<const unsigned short*>(p.ffn2)) +
                              static_cast<size_t>(tile.expert) * H * I;
   TileRows rows;
-  rows.wbase = reinterpret_cast<const unsigned char*>(w2);
   rows.tbase = reinterpret_cast<const unsigned char*>(
       uni(reinterpret_cast<const unsigned short*>(p.h)) + static_cast<size_t>(tile.row0) * I);
+  rows.wpacked = uni(p.ffn2_packed != nullptr ? 1 : 0) != 0;
+  rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
 #pragma unroll
   for (int q = 0; q < LQ; ++q) {
     const int row = stage_row(q);
-    rows.woff[q] = static_cast<unsigned>(n0 + row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
+    if (rows.wpacked) {
+      // stage block B (16 rows of W2): the packed task of 64 output columns holds its blocks 0..3
+      const int B = uni(static_cast<int>(threadIdx.x >> 6)) * LQ + q;
+      const size_t task = static_cast<size_t>(tile.expert) * (H / 64) + (n0 / 64 + (B >> 2));
+      rows.wbase[q] = uni(reinterpret_cast<const unsigned char*>(p.ffn2_packed)) +
+                      task * (static_cast<size_t>(I / 32) * 4096) + (B & 3) * 1024;
+      rows.woff[q] = (threadIdx.x & 63) * 16;
+    } else {
+      rows.wbase[q] = reinterpret_cast<const unsigned char*>(w2);
+      rows.woff[q] = static_cast<unsigned>(n0 + row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
+    }
     rows.toff[q] = static_cast<unsigned>(min(row, tile.rows - 1)) * static_cast<unsigned>(I * 2) +
                    stage_chunk_bytes(row);
   }

@@ -134,6 +134,13 @@ def test_tiled_variant_forced(shape):
             assert torch.allclose(out.float(), out2.float(), rtol=2e-2, atol=1e-3)
         finally:
             other.close()
+        # the tiled variant reading the packed weight copy computes the same bits
+        packed = GpuCase(cfg, seed=T + E, sched=_lib.SCHED_TILED, inputs=case.inp, pack_weights=True)
+        try:
+            assert packed.launcher.sched_for(T) == _lib.SCHED_TILED
+            assert torch.equal(packed.run(), out)
+        finally:
+            packed.close()
     finally:
         case.close()
 
