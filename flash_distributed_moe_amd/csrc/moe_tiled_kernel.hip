@@ -439,7 +439,9 @@ struct TileRows {
   const unsigned char* wbase[LQ];  // uniform: where this wave's weight load q starts at k-step 0
   const unsigned char* tbase;      // uniform: tokens, or this tile's h rows
   unsigned wkstride;               // uniform: bytes from one k-step's weights to the next
+  unsigned tkstride;               // uniform: the same for the token rows
   bool wpacked;                    // uniform: weight blocks are 1 KiB runs
+  bool tpacked;                    // uniform: so are the token blocks (the down projection's h rows)
   unsigned woff[LQ];               // byte offset of this lane's 16 bytes of weight load q
   unsigned toff[LQ];               // token stage: this lane's chunk of stage row wave*16*LQ+q*16+(lane>>2)
 };
@@ -487,7 +489,7 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
     if (q < LQ) {
       load_to_lds(rows.woff[q], rows.wbase[q] + static_cast<size_t>(src) * rows.wkstride, st + q * 1024);
     } else {
-      load_to_lds(rows.toff[q - LQ], rows.tbase + static_cast<size_t>(src) * (TK * 2),
+      load_to_lds(rows.toff[q - LQ], rows.tbase + static_cast<size_t>(src) * rows.tkstride,
                   st + TN * TK * 2 + (q - LQ) * 1024);
     }
   };
@@ -509,8 +511,12 @@ __device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, co
     const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? ra0 : ra1);
     if (JMAX > 0) f.a[i] = *reinterpret_cast<const uint4*>(st + wblk[i] * 64);
   };
+  const int pk0 = (r32 >> 4) * 1024 + ((kq * 16 + (r32 & 15)) << 4);
+  const int pk1 = (r32 >> 4) * 1024 + (((2 + kq) * 16 + (r32 & 15)) << 4);
+  const int rb0 = rows.tpacked ? pk0 : rd0;
+  const int rb1 = rows.tpacked ? pk1 : rd1;
   auto read_b = [&](Frags& f, int ks, int kk, int j) {
-    const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? rd0 : rd1);
+    const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? rb0 : rb1);
     if (j < JMAX) f.b[j] = *reinterpret_cast<const uint4*>(st + TN * TK * 2 + (tok0 + j * 32) * 64);
   };
   auto read = [&](Frags& f, int ks, int kk) {
@@ -622,9 +628,14 @@ __device__ __forceinline__ unsigned stage_chunk_bytes(int row) {
   return static_cast<unsigned>(((threadIdx.x & 3) ^ ((row >> 2) & 3)) << 4);
 }
 
+// h of the tiled variant: row tile m owns 256 rows x I, stored the way the down
+// projection's loads want them: [k-step of 32 columns][16-row block][chunk 0..3][row 0..15][16 B],
+// so a block of a k-step is one 1 KiB run.
+__device__ __forceinline__ size_t tiled_h_tile_bytes(int I) { return static_cast<size_t>(TM) * I * 2; }
+
 // gate/up: h[row, n0 .. n0+128) for one row tile
 // (test/singleGPU/cpp/moe/reference/refExpertFFN1.h:51-65).
-__device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& tile_in, int nblk) {
+__device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& tile_in, int m, int nblk) {
   const int H = uni(p.H), I = uni(p.I), K = uni(p.K);
   TileDesc tile;
   tile.expert = uni(tile_in.expert);
@@ -636,6 +647,8 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
   TileRows rows;
   rows.wpacked = uni(p.ffn1_packed != nullptr ? 1 : 0) != 0;
   rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
+  rows.tkstride = static_cast<unsigned>(TK * 2);
+  rows.tpacked = false;
   rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
 #pragma unroll
   for (int q = 0; q < LQ; ++q) {
@@ -664,8 +677,9 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
   const int tok0 = wm * (32 * WJ);
   const int jmax = uni(min(WJ, max(0, (tile.rows - tok0 + 31) / 32)));
   const bool tokl = wave * (16 * LQ) < tile.rows;  // some of the token rows this wave loads exist
-  unsigned short* h = uni(reinterpret_cast<unsigned short*>(p.h)) +
-                      static_cast<size_t>(tile.row0) * I + n0 + wn * 64;
+  // this wave's 64 columns are k-steps (n0 + 64*wn)/32 and the next of the tile's h
+  unsigned char* h = uni(reinterpret_cast<unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I) +
+                     static_cast<size_t>((n0 + wn * 64) / 32) * (TM * 64);
   f32x16 acc[4][WJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -701,11 +715,13 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
       lds_wave_sync();
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
-        const int rr = it * 8 + (lane >> 3), cc = (lane & 7) * 8;
+        // one 1 KiB run: k-step it / 2 of this wave's two, 16-row block it % 2 of this token block
+        const int ksl = it >> 1, b16 = it & 1;
+        const int rr = b16 * 16 + (lane & 15), cc = ksl * 32 + (lane >> 4) * 8;
         const int trow = tok0 + j * 32 + rr;
         const uint4 v = *reinterpret_cast<const uint4*>(slab + rr * SLD + cc);
         if (trow < tile.rows)
-          st16_through(h + static_cast<size_t>(trow) * I + cc, v);
+          st16_through(h + static_cast<size_t>(ksl) * (TM * 64) + ((tok0 + j * 32) / 16 + b16) * 1024 + lane * 16, v);
       }
       lds_wave_sync();
     }
@@ -714,7 +730,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
 
 // down: y[t*K+slot, n0 .. n0+256) = w * (h[row] . W2[e]^T)
 // (refFullMoe.h:58-65, src/hip/kernel/tasks/ffn2Task.h:37-40).
-__device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& tile_in, int nblk) {
+__device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& tile_in, int m, int nblk) {
   const int H = uni(p.H), I = uni(p.I);
   TileDesc tile;
   tile.expert = uni(tile_in.expert);
@@ -724,8 +740,9 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
   const unsigned short* w2 = uni(reinterpret_cast<const unsigned short*>(p.ffn2)) +
                              static_cast<size_t>(tile.expert) * H * I;
   TileRows rows;
-  rows.tbase = reinterpret_cast<const unsigned char*>(
-      uni(reinterpret_cast<const unsigned short*>(p.h)) + static_cast<size_t>(tile.row0) * I);
+  rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I);
+  rows.tkstride = static_cast<unsigned>(TM * 64);
+  rows.tpacked = true;
   rows.wpacked = uni(p.ffn2_packed != nullptr ? 1 : 0) != 0;
   rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
 #pragma unroll
@@ -742,8 +759,9 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
       rows.wbase[q] = reinterpret_cast<const unsigned char*>(w2);
       rows.woff[q] = static_cast<unsigned>(n0 + row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
     }
-    rows.toff[q] = static_cast<unsigned>(min(row, tile.rows - 1)) * static_cast<unsigned>(I * 2) +
-                   stage_chunk_bytes(row);
+    // token stage block wave*LQ + q is one run of the tile's h (rows past the tile's
+    // end were never written; their products are dropped)
+    rows.toff[q] = static_cast<unsigned>((uni(static_cast<int>(threadIdx.x >> 6)) * LQ + q) * 1024 + (threadIdx.x & 63) * 16);
   }
   const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int wn = wave & 1, wm = wave >> 1;
@@ -986,7 +1004,7 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
         const unsigned m = lo + j / nt1;
         if (p.trace) t_ready = wall_clock64();
         const TileDesc tile = ld_tile(&p.mtiles[m]);
-        tiled_gateup_task(p, tile, static_cast<int>(j % nt1));
+        tiled_gateup_task(p, tile, static_cast<int>(m), static_cast<int>(j % nt1));
         wg_arrive<false>(&p.g1_done[m].v, &sh);
         trace(t_dyn0 + lo * nt1 + j, 3, m, t_fetch, t_ready);
       } else {
@@ -996,7 +1014,7 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
         if (ok) {
           if (p.trace) t_ready = wall_clock64();
           const TileDesc tile = ld_tile(&p.mtiles[m]);
-          tiled_down_task(p, tile, static_cast<int>(jj % nt2));
+          tiled_down_task(p, tile, static_cast<int>(m), static_cast<int>(jj % nt2));
           if (wg_arrive<false>(&ctl->g2_done.v, &sh) == n2_total - 1u) wg_broadcast_flag(p, FLAG_G2);
           trace(t_dyn0 + nm * nt1 + lo * nt2 + jj, 4, m, t_fetch, t_ready);
         }
