@@ -43,10 +43,11 @@ enum { FLASH_MOE_F32 = 0, FLASH_MOE_BF16 = 1 };
 enum { FLASH_MOE_SCHED_AUTO = 0, FLASH_MOE_SCHED_STREAM = 1, FLASH_MOE_SCHED_TILED = 2 };
 
 /* FLASH_MOE_FLAG_PACK_WEIGHTS: at create the expert weights are copied once into
- * a layout that the streaming (small-batch) variant reads front to back, which
- * is what HBM likes best; costs a second copy of the expert weights in device
- * memory. The caller's tensors stay the external format and are still what the
- * tiled variant reads; after changing them call flashMoeRefreshWeights. */
+ * a layout of contiguous 1 KiB runs (16 rows x 32 k) that the streaming
+ * (small-batch) variant reads front to back and the tiled variant loads as
+ * whole cache lines; costs a second copy of the expert weights in device
+ * memory. The caller's tensors stay the external format and are no longer read
+ * by launches; after changing them call flashMoeRefreshWeights. */
 enum { FLASH_MOE_FLAG_PACK_WEIGHTS = 1 };
 
 typedef struct FlashMoeLayerDesc {
