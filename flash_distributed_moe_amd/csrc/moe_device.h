@@ -202,12 +202,8 @@ __device__ __forceinline__ uint4 ld16_agent(const CoherentBuffer& b, unsigned of
 // 16 bytes that are used once (expert weights): marked non-temporal, so that
 // they do not push the token rows and the routing tables out of the L2
 __device__ __forceinline__ uint4 ld16_once(const void* p) {
-#ifdef FMOE_NO_NT
-  return ld16(p);
-#else
   const u32x4 v = __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x4*>(p)));
   return make_uint4(v.x, v.y, v.z, v.w);
-#endif
 }
 __device__ __forceinline__ void st16(void* p, const u32x4& v) {
   *as_global(reinterpret_cast<u32x4*>(p)) = v;

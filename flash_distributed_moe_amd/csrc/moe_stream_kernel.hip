@@ -29,9 +29,6 @@
 // (src/hip/kernel/tasks/*.h) and its queue (src/hip/taskSystem/*.h).
 #include "moe_device.h"
 
-#ifndef FMOE_COH_B
-#define FMOE_COH_B true
-#endif
 namespace fmoe {
 
 // --------------------------------------------------------------------- router
@@ -74,10 +71,7 @@ __device__ __noinline__ void router_dot_task(const Params& p, int tg, int eg) {
   const elem* tokens = reinterpret_cast<const elem*>(p.tokens);
 
   // PF k-chunks of global loads are in flight ahead of the chunk being consumed
-#ifndef FMOE_ROUTER_PF
-#define FMOE_ROUTER_PF 1
-#endif
-  constexpr int PF = EPV == 8 ? FMOE_ROUTER_PF : (FMOE_ROUTER_PF + 1) / 2;
+  constexpr int PF = 1;  // deeper prefetch measured slower (registers)
   uint4 wr[PF][NLD], xr[PF][NLD];
   auto issue = [&](uint4(&wq)[NLD], uint4(&xq)[NLD], int c0) {  // global -> registers
     if (c0 >= H) return;
@@ -551,10 +545,7 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
 // loads of 16 bytes per lane.
 template <int NA, int RB>
 struct RoundSteps {
-#ifndef FMOE_U1
-#define FMOE_U1 8
-#endif
-  static constexpr int value = RB == 1 ? (NA <= 2 ? 2 * FMOE_U1 : FMOE_U1) : (RB == 2 ? (NA <= 2 ? 8 : 4) : 4);
+  static constexpr int value = RB == 1 ? (NA <= 2 ? 16 : 8) : (RB == 2 ? (NA <= 2 ? 8 : 4) : 4);
 };
 
 // -------------------------------------------------------------------- gate/up
@@ -782,7 +773,7 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
   // The h rows are read at agent scope: two gate/up tasks, possibly on different
   // XCDs, each write half of a 128-byte line of h, so this XCD's L2 may hold a
   // line one of its own tasks wrote before the other half existed.
-  const bool ok = stream_mma<DT, NA, RB, U, FMOE_COH_B>(ap, bp, p.I / (4 * EPV), astep, acc, [&] {
+  const bool ok = stream_mma<DT, NA, RB, U, true>(ap, bp, p.I / (4 * EPV), astep, acc, [&] {
     return wave_wait_ge(dep, dep_target, p.ctl, p.spin_limit);
   }, hbase, hbytes);
   if (!ok) return false;
