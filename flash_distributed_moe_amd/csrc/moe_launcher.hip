@@ -300,8 +300,12 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
 }
 
 // The tiled variant needs bf16, tile-aligned shapes and token rows it can
-// address with 32-bit byte offsets; AUTO takes it once an expert sees about 48
-// rows on average.
+// address with 32-bit byte offsets. AUTO takes it once an expert sees about 24
+// rows on average when the packed weight copy exists (30B shape, us, streaming /
+// tiled: T=384 338 / 340, T=512 379 / 342; 235B shape: T=256 970 / 1018, T=512
+// 1119 / 1048), and from about 4 rows when the weights are read in the caller's
+// row-major layout, which the streaming variant reads poorly (30B: T=64 359 /
+// 352, T=128 411 / 358).
 static bool tiled_eligible(const FlashMoeLayerDesc& d, int tokens_num) {
   return d.dtype == FLASH_MOE_BF16 && d.hidden % 256 == 0 && d.intermediate % 128 == 0 &&
          tokens_num <= fmoe::tiled_max_tokens() &&
@@ -315,7 +319,8 @@ int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num) {
   if (!tiled_eligible(d, tokens_num)) return FLASH_MOE_SCHED_STREAM;
   if (d.sched == FLASH_MOE_SCHED_TILED) return FLASH_MOE_SCHED_TILED;
   const long long rows = static_cast<long long>(tokens_num) * d.top_k;
-  return rows >= 48ll * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
+  const bool packed = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
+  return rows >= (packed ? 24ll : 4ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
 }
 
 int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int tokens_num,

@@ -96,7 +96,7 @@ def test_nan_and_all_equal_logits(name):
         case.close()
 
 
-@pytest.mark.parametrize("name,T,sched", [("qwen3_30b_decode", 64, 0), ("qwen3_30b_decode", 512, 2)])
+@pytest.mark.parametrize("name,T,sched", [("qwen3_30b_decode", 64, 1), ("qwen3_30b_decode", 512, 2)])
 def test_device_wait_limit_is_reported_and_cleared(name, T, sched):
     """With a wait limit of 100 ns every dependency wait that has to wait at all
     gives up: the kernel ends normally, flashMoeStatus reports bit 1 and re-arms

@@ -27,12 +27,12 @@ def check_perm_properties(r, T, k, E):
     assert np.all(inner | boundary)                   # ascending (token, slot) inside a segment
 
 
-def run_full(name, sample, T=None):
+def run_full(name, sample, T=None, pack_weights=False):
     cfg = synth.CONFIGS[name]
     if T is not None:
         cfg = cfg.replace(T=T)
-    print("full config", cfg.name, "T", cfg.T, flush=True)
-    case = GpuCase(cfg)
+    print("full config", cfg.name, "T", cfg.T, "packed" if pack_weights else "caller's layout", flush=True)
+    case = GpuCase(cfg, pack_weights=pack_weights)
     try:
         x = case.inp["tokens"]
         out = case.run()
@@ -49,12 +49,15 @@ def run_full(name, sample, T=None):
         case.close()
 
 
-def test_qwen3_30b_prefill():
-    run_full("qwen3_30b_prefill", sample=48)
+@pytest.mark.parametrize("pack_weights", [False, True])
+def test_qwen3_30b_prefill(pack_weights):
+    run_full("qwen3_30b_prefill", sample=48, pack_weights=pack_weights)
 
 
-def test_qwen3_235b_t256():
-    run_full("qwen3_235b_t256", sample=24)
+@pytest.mark.parametrize("pack_weights", [False, True])
+def test_qwen3_235b_t256(pack_weights):
+    # AUTO: the tiled variant on the caller's layout, the streaming one on the packed copy
+    run_full("qwen3_235b_t256", sample=24, pack_weights=pack_weights)
 
 
 def test_qwen3_235b_t4096():

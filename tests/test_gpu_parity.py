@@ -11,7 +11,7 @@ from tests.moe_case import GpuCase
 pytestmark = pytest.mark.gpu
 
 
-def run_case(cfg, seed=7907, sched=_lib.SCHED_AUTO, sample=None, inplace=False):
+def run_case(cfg, seed=7907, sched=_lib.SCHED_STREAM, sample=None, inplace=False):
     print("case", cfg.name, "T", cfg.T, "H", cfg.H, "E", cfg.E, "k", cfg.k, "I", cfg.I,
           cfg.dtype, "seed", seed, "sched", sched, flush=True)
     case = GpuCase(cfg, seed, sched)
@@ -50,19 +50,23 @@ def test_tiny_f32_matches_golden(golden_dir):
         case.close()
 
 
-@pytest.mark.parametrize("seed", [7907, 1, 2])
-def test_qwen3_30b_decode(seed):
-    run_case(synth.CONFIGS["qwen3_30b_decode"], seed=seed)
+# AUTO on the caller's weight layout takes the tiled variant from T*k >= 4*E on
+@pytest.mark.parametrize("seed,sched", [(7907, _lib.SCHED_STREAM), (1, _lib.SCHED_STREAM),
+                                        (2, _lib.SCHED_STREAM), (7907, _lib.SCHED_AUTO)])
+def test_qwen3_30b_decode(seed, sched):
+    run_case(synth.CONFIGS["qwen3_30b_decode"], seed=seed, sched=sched)
 
 
-def test_qwen3_30b_decode_inplace():
-    run_case(synth.CONFIGS["qwen3_30b_decode"], inplace=True)
+@pytest.mark.parametrize("sched", [_lib.SCHED_STREAM, _lib.SCHED_AUTO])
+def test_qwen3_30b_decode_inplace(sched):
+    run_case(synth.CONFIGS["qwen3_30b_decode"], inplace=True, sched=sched)
 
 
+@pytest.mark.parametrize("sched", [_lib.SCHED_STREAM, _lib.SCHED_AUTO])
 @pytest.mark.parametrize("T", [1, 3, 17, 65, 130])
-def test_ragged_token_counts_bf16(T):
+def test_ragged_token_counts_bf16(T, sched):
     cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=T, name="ragged")
-    run_case(cfg, seed=T)
+    run_case(cfg, seed=T, sched=sched)
 
 
 @pytest.mark.parametrize("shape", [
@@ -89,7 +93,7 @@ def test_router_bias_hot_experts_small():
 def test_relaunch_and_smaller_batch():
     """Counters return to zero by themselves: launch twice, then a smaller batch."""
     cfg = synth.CONFIGS["qwen3_30b_decode"]
-    case = GpuCase(cfg)
+    case = GpuCase(cfg, sched=_lib.SCHED_STREAM)
     try:
         x = case.inp["tokens"]
         a = case.run()
@@ -172,9 +176,9 @@ def test_packed_weights_equal_unpacked(name, T):
     """The packed second copy of the expert weights changes where bytes are read
     from, not what is computed."""
     cfg = synth.CONFIGS[name].replace(T=T)
-    a = GpuCase(cfg, seed=11)
+    a = GpuCase(cfg, seed=11, sched=_lib.SCHED_STREAM)
     try:
-        b = GpuCase(cfg, seed=11, inputs=a.inp, pack_weights=True)
+        b = GpuCase(cfg, seed=11, sched=_lib.SCHED_STREAM, inputs=a.inp, pack_weights=True)
         try:
             out_a, out_b = a.run(), b.run()
             assert torch.equal(out_a, out_b)
