@@ -337,6 +337,138 @@ __device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
   }
 }
 
+// The same for 16 tokens, used while that still gives every workgroup at most one
+// router task (T <= 16 x workgroups): with 32-token tasks half of the CUs or more
+// would sit through the router idle. The chains run on V_MFMA_F32_16X16X4_F32
+// (which also adds its products in k order, one rounding each): wave w carries
+// the 16 tokens x experts 16w..16w+15 of the slab. All eight waves load: 64 k of
+// the 16 token rows and the 128 expert rows per stage, rows 144 bytes apart as
+// above. Lane l multiplies row l % 16 of both operands at k = 4*s + l/16: of the
+// eight bf16 a 16-byte read brings, elements l/16 and 4 + l/16, each moved into
+// the upper half of a zero word by one byte permute.
+constexpr int RT16_TOK = 16;
+__device__ __forceinline__ void load_to_lds_addr(const unsigned char* addr, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(addr), "s"(lds_addr)
+               : "memory");
+}
+
+__device__ __noinline__ void tiled_router16_task(const Params& p, int blk) {
+  const int T = uni(p.T), E = uni(p.E), H = uni(p.H);
+  const unsigned char* tokens = uni(reinterpret_cast<const unsigned char*>(p.tokens));
+  const unsigned char* gate = uni(reinterpret_cast<const unsigned char*>(p.gate));
+  const float* bias = uni(p.bias);
+  unsigned* keys = reinterpret_cast<unsigned*>(lds_raw + RT_STAGES * RT_STAGE_BYTES);  // [RT16_TOK][MAX_EXPERTS]
+  double* sel = reinterpret_cast<double*>(keys + RT_TOK * MAX_EXPERTS);                // WAVES x MAX_TOPK
+  const unsigned lds_addr = uni(static_cast<unsigned>(
+      reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
+  const int tid = threadIdx.x;
+  const int wave = uni(tid >> 6), lane = tid & 63;
+  const int t0 = uni(blk) * RT16_TOK;
+  const int nsteps = H >> 6;
+  // slot g of a stage (16 bytes): position g % 9 of row g / 9 (position 8 is padding);
+  // rows 0..15 are the tokens, 16..143 the experts of the slab; slots past the last row repeat it
+  constexpr int NL = 3;  // loads per wave and stage: 1536 slots >= 144 rows x 9
+  constexpr int NROWS = RT16_TOK + 128;
+  static_assert(NROWS * 9 <= WAVES * NL * 64 && WAVES * NL * 1024 == RT_STAGE_BYTES, "router stage");
+  const int r16 = lane & 15, kq = lane >> 4;
+  const unsigned pick = kq == 0 ? 0x01000C0Cu : kq == 1 ? 0x03020C0Cu : kq == 2 ? 0x05040C0Cu : 0x07060C0Cu;
+  const int xoff = r16 * RT_ROW_BYTES;
+  const int woff = (RT16_TOK + 16 * wave + r16) * RT_ROW_BYTES;
+  for (int e0 = 0; e0 < E; e0 += 128) {
+    const unsigned char* src[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int g = (wave * NL + i) * 64 + lane;
+      const int row = min(g / 9, NROWS - 1);
+      const int pos = min(g % 9, 7);
+      const unsigned char* base =
+          row < RT16_TOK ? tokens + static_cast<size_t>(min(t0 + row, T - 1)) * H * 2
+                         : gate + static_cast<size_t>(min(e0 + row - RT16_TOK, E - 1)) * H * 2;
+      src[i] = base + pos * 16;
+    }
+    auto issue = [&](int step) {  // past the last step: the last one again, into a stage nobody reads
+      const size_t koff = static_cast<size_t>(min(step, nsteps - 1)) * 128;
+      const unsigned st = lds_addr + (step & (RT_STAGES - 1)) * RT_STAGE_BYTES + wave * (NL * 1024);
+#pragma unroll
+      for (int i = 0; i < NL; ++i) load_to_lds_addr(src[i] + koff, st + i * 1024);
+    };
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    // Operands of half a stage (32 k): four 16-byte chunks of both rows. While the 8
+    // matrix instructions of one half run, the next half is read, one chunk of both
+    // rows after each pair; the scheduling barriers keep the reads from being
+    // gathered in front of their first use, where their latency would be exposed.
+    struct Half {
+      uint4 a[4], w[4];
+    };
+    auto read_chunk = [&](Half& h, const unsigned char* hb, int c4) {
+      h.a[c4] = *reinterpret_cast<const uint4*>(hb + xoff + 16 * c4);
+      h.w[c4] = *reinterpret_cast<const uint4*>(hb + woff + 16 * c4);
+    };
+    auto chain_and_read = [&](const Half& h, Half& nx, const unsigned char* nb) {
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
+            __uint_as_float(__builtin_amdgcn_perm(h.a[c4].y, h.a[c4].x, pick)),
+            __uint_as_float(__builtin_amdgcn_perm(h.w[c4].y, h.w[c4].x, pick)), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
+            __uint_as_float(__builtin_amdgcn_perm(h.a[c4].w, h.a[c4].z, pick)),
+            __uint_as_float(__builtin_amdgcn_perm(h.w[c4].w, h.w[c4].z, pick)), acc, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_chunk(nx, nb, c4);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+#pragma unroll
+    for (int st = 0; st < RT_STAGES; ++st) issue(st);
+    wait_vm<(RT_STAGES - 1) * NL>();
+    __builtin_amdgcn_s_barrier();  // stage 0 is in
+    asm volatile("" ::: "memory");
+    Half h0, h1;
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4) read_chunk(h0, lds_raw, c4);
+    for (int st = 0; st < nsteps; ++st) {
+      chain_and_read(h0, h1, lds_raw + (st & (RT_STAGES - 1)) * RT_STAGE_BYTES + 64);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave no longer reads stage st
+      wait_vm<(RT_STAGES - 2) * NL>();                    // its loads of stage st+1 are in
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      issue(st + RT_STAGES);
+      // after the last step this reads a stage that is being refilled; the values are never used
+      chain_and_read(h1, h0, lds_raw + ((st + 1) & (RT_STAGES - 1)) * RT_STAGE_BYTES);
+    }
+    wait_vm<0>();                  // nothing may land in a stage after this slab
+    __builtin_amdgcn_s_barrier();  // the stages may be refilled for the next slab
+    asm volatile("" ::: "memory");
+    // acc[v] of lane l: token 4*(l/16) + v, expert e0 + 16*wave + l%16
+    const int e = e0 + 16 * wave + r16;
+    const float bv = (bias != nullptr && e < E) ? as_global(bias)[e] : 0.0f;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float x = acc[v];
+      if (bias != nullptr) x = __fadd_rn(x, bv);
+      if (e < MAX_EXPERTS) keys[(4 * kq + v) * MAX_EXPERTS + e] = ordered_bits(x, e < E);
+    }
+  }
+  __syncthreads();
+  // selection: two tokens per wave
+  double* lex = sel + wave * MAX_TOPK;
+  for (int i = 0; i < RT16_TOK / WAVES; ++i) {
+    const int tl = wave * (RT16_TOK / WAVES) + i;
+    const int t = t0 + tl;
+    if (t < T) {
+      unsigned val[MAX_EXPERTS / 64];
+#pragma unroll
+      for (int j = 0; j < MAX_EXPERTS / 64; ++j) {
+        const int e = lane + 64 * j;
+        val[j] = e < E ? keys[tl * MAX_EXPERTS + e] : 0u;
+      }
+      router_select_max(p, t, val, lex);
+    }
+  }
+}
+
 // ----------------------------------------------------------------------- scan
 // Same tables as the streaming variant's scan, in two steps. Expert scan: one
 // wave per expert walks the expert's mask words 64 at a time and writes the
@@ -911,12 +1043,15 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
   __syncthreads();
   Control* ctl = p.ctl;
   const unsigned T = static_cast<unsigned>(p.T);
-  const unsigned n_rt = (T + RT_TOK - 1u) / RT_TOK;
+  const unsigned n_sc = (T + RT_TOK - 1u) / RT_TOK;  // scatter tasks
+  // router tasks: of 16 tokens while every workgroup still gets at most one
+  const bool router16 = (T + RT16_TOK - 1u) / RT16_TOK <= gridDim.x;
+  const unsigned n_rt = router16 ? (T + RT16_TOK - 1u) / RT16_TOK : n_sc;
   const unsigned n_es = (static_cast<unsigned>(p.E) + SCAN_EXPERTS - 1u) / SCAN_EXPERTS;
   const unsigned t_escan0 = n_rt;
   const unsigned t_scan = n_rt + n_es;
   const unsigned t_scatter0 = t_scan + 1u;
-  const unsigned t_dyn0 = t_scatter0 + n_rt;
+  const unsigned t_dyn0 = t_scatter0 + n_sc;
   const unsigned nt1 = static_cast<unsigned>(p.I / G1_COLS);
   const unsigned nt2 = static_cast<unsigned>(p.H / TN);
   const unsigned ncmb = (T + CMB_TOK - 1u) / CMB_TOK;
@@ -950,7 +1085,11 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
     long long t_ready = 0;
     if (tk < n_rt) {
       if (p.trace) t_ready = wall_clock64();
-      tiled_router_task(p, static_cast<int>(tk));
+      if (router16) {
+        tiled_router16_task(p, static_cast<int>(tk));
+      } else {
+        tiled_router_task(p, static_cast<int>(tk));
+      }
       wg_arrive<false>(&ctl->router_done.v, &sh);
       trace(tk, 0, tk, t_fetch, t_ready);
     } else if (tk < t_scan) {
@@ -973,7 +1112,7 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
       if (ok) {
         if (p.trace) t_ready = wall_clock64();
         tiled_scatter_task(p, static_cast<int>(tk - t_scatter0));
-        if (wg_arrive<false>(&ctl->perm_done.v, &sh) == n_rt - 1u) wg_broadcast_flag(p, FLAG_PERM);
+        if (wg_arrive<false>(&ctl->perm_done.v, &sh) == n_sc - 1u) wg_broadcast_flag(p, FLAG_PERM);
         trace(tk, 2, tk - t_scatter0, t_fetch, t_ready);
       }
     }
