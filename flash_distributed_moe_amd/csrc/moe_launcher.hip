@@ -96,9 +96,9 @@ Layout make_layout(const FlashMoeLayerDesc& d) {
   L.row_w = take(sizeof(float) * rows);
   L.mtiles = take(sizeof(fmoe::TileDesc) * L.max_mtiles);
   // h: [rows, I] routed, or [E, 64, I] when small batches run gate/up densely
-  // (the tiled variant keeps 256 rows per row tile, and an expert's last tile is partial)
+  // (the tiled variant reserves 320 rows per row tile, and an expert's last tile is partial)
   const size_t h_rows = std::max<size_t>({rows, static_cast<size_t>(d.experts) * 64,
-                                          (rows / 256 + static_cast<size_t>(d.experts) + 1) * 256});
+                                          (rows / 256 + static_cast<size_t>(d.experts) + 1) * 320});
   L.h = take(esz * h_rows * d.intermediate);
   L.y = take(sizeof(float) * rows * d.hidden);
   const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;

@@ -47,7 +47,15 @@ constexpr int CMB_TOK = 8;         // tokens per combine task
 
 constexpr int TILE_LDS_BYTES = STAGES * STAGE_BYTES;  // 131072
 constexpr int ROUTER_LDS_BYTES = 4 * 24576 + RT_TOK * MAX_EXPERTS * 4 + WAVES * MAX_TOPK * 8;
-constexpr int TILED_LDS_BYTES = TILE_LDS_BYTES > ROUTER_LDS_BYTES ? TILE_LDS_BYTES : ROUTER_LDS_BYTES;
+// Tall row tiles: an expert's last 1..TALL_EXTRA rows join its last full tile instead of
+// costing a pass of their own over the expert's weights.
+constexpr int TALL_EXTRA = 64;
+constexpr int TALL_TM = TM + TALL_EXTRA;                       // 320 token rows
+constexpr int TALL_STAGE_BYTES = (TN + TALL_TM) * TK * 2;      // 36 KiB: weight rows, then token rows
+constexpr int TALL_LDS_BYTES = STAGES * TALL_STAGE_BYTES;      // 147456
+constexpr int HT_ROWS = TALL_TM;                               // rows a row tile owns in h
+constexpr int TILED_LDS_BYTES_0 = TILE_LDS_BYTES > ROUTER_LDS_BYTES ? TILE_LDS_BYTES : ROUTER_LDS_BYTES;
+constexpr int TILED_LDS_BYTES = TILED_LDS_BYTES_0 > TALL_LDS_BYTES ? TILED_LDS_BYTES_0 : TALL_LDS_BYTES;
 
 extern __shared__ __align__(16) unsigned char lds_raw[];
 
@@ -508,16 +516,19 @@ __device__ __noinline__ void tiled_scan_task(const Params& p) {
       const int c = e < r.E ? ldc(&r.expert_count[e]) : 0;
       const int incl = wave_inclusive_scan(c);
       const int off = base + incl - c;
-      const int nt = (c + TM - 1) / TM;
+      // a tail of at most TALL_EXTRA rows joins the last full tile (a tall tile)
+      const bool tall = c > TM && (c % TM) != 0 && (c % TM) <= TALL_EXTRA;
+      const int nt = tall ? c / TM : (c + TM - 1) / TM;
       const int tincl = wave_inclusive_scan(nt);
       const int toff = tile_base + tincl - nt;
       if (e < r.E) {
         stc(&r.expert_offset[e], off);
         for (int i = 0; i < nt; ++i) {
           if (toff + i < r.max_mtiles) {
+            const int tr = (tall && i == nt - 1) ? c - i * TM : min(TM, c - i * TM);
             stc16(&r.mtiles[toff + i],
                   make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + i * TM),
-                             static_cast<unsigned>(min(TM, c - i * TM)), 0u));
+                             static_cast<unsigned>(tr), 0u));
           }
         }
       }
@@ -760,10 +771,10 @@ __device__ __forceinline__ unsigned stage_chunk_bytes(int row) {
   return static_cast<unsigned>(((threadIdx.x & 3) ^ ((row >> 2) & 3)) << 4);
 }
 
-// h of the tiled variant: row tile m owns 256 rows x I, stored the way the down
+// h of the tiled variant: row tile m owns HT_ROWS rows x I, stored the way the down
 // projection's loads want them: [k-step of 32 columns][16-row block][chunk 0..3][row 0..15][16 B],
 // so a block of a k-step is one 1 KiB run.
-__device__ __forceinline__ size_t tiled_h_tile_bytes(int I) { return static_cast<size_t>(TM) * I * 2; }
+__device__ __forceinline__ size_t tiled_h_tile_bytes(int I) { return static_cast<size_t>(HT_ROWS) * I * 2; }
 
 // gate/up: h[row, n0 .. n0+128) for one row tile
 // (test/singleGPU/cpp/moe/reference/refExpertFFN1.h:51-65).
@@ -811,7 +822,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
   const bool tokl = wave * (16 * LQ) < tile.rows;  // some of the token rows this wave loads exist
   // this wave's 64 columns are k-steps (n0 + 64*wn)/32 and the next of the tile's h
   unsigned char* h = uni(reinterpret_cast<unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I) +
-                     static_cast<size_t>((n0 + wn * 64) / 32) * (TM * 64);
+                     static_cast<size_t>((n0 + wn * 64) / 32) * (HT_ROWS * 64);
   f32x16 acc[4][WJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -853,7 +864,7 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
         const int trow = tok0 + j * 32 + rr;
         const uint4 v = *reinterpret_cast<const uint4*>(slab + rr * SLD + cc);
         if (trow < tile.rows)
-          st16_through(h + static_cast<size_t>(ksl) * (TM * 64) + ((tok0 + j * 32) / 16 + b16) * 1024 + lane * 16, v);
+          st16_through(h + static_cast<size_t>(ksl) * (HT_ROWS * 64) + ((tok0 + j * 32) / 16 + b16) * 1024 + lane * 16, v);
       }
       lds_wave_sync();
     }
@@ -873,7 +884,7 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
                              static_cast<size_t>(tile.expert) * H * I;
   TileRows rows;
   rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I);
-  rows.tkstride = static_cast<unsigned>(TM * 64);
+  rows.tkstride = static_cast<unsigned>(HT_ROWS * 64);
   rows.tpacked = true;
   rows.wpacked = uni(p.ffn2_packed != nullptr ? 1 : 0) != 0;
   rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
@@ -963,6 +974,335 @@ __device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& ti
     }
   }
 }
+
+// ------------------------------------------------------------ tall row tiles
+// A row tile of 257..320 rows (an expert's last full tile plus its short tail):
+// one pass over the expert's weights instead of two. Waves are laid out 4 (64
+// weight rows, two blocks) x 2 (160 token rows, five blocks): 160 accumulator
+// registers per lane. A stage holds 256 weight rows and 320 token rows (36 KiB);
+// every wave loads two weight blocks, and token blocks wave, wave + 8 and (waves
+// 0..3) wave + 16 of the twenty 16-row blocks. Otherwise as tile_gemm_j.
+struct TallRows {
+  const unsigned char* wbase[LQ];
+  const unsigned char* tbase;
+  unsigned wkstride, tkstride;
+  bool wpacked, tpacked;
+  unsigned woff[LQ];
+  unsigned toff[3];
+};
+struct TallFrags {
+  uint4 a[2];  // weight blocks
+  uint4 b[5];  // token blocks
+};
+
+// NTB: token blocks of this wave that are computed (4 or 5); NTL: its token loads per stage (2 or 3)
+template <int NTB, int NTL>
+__device__ __forceinline__ void tall_gemm(const TallRows& rows, int ksteps, const int (&wblk)[2], int tok0,
+                                          f32x16 (&acc)[2][5]) {
+  constexpr int NLD = LQ + NTL;  // this wave's loads per stage
+  static_assert(LQ == 2 && NLD <= 5, "tall tiles are written for eight waves");
+  const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
+  const int r32 = lane & 31, kq = lane >> 5;
+  const unsigned char* lds = lds_raw;
+  const unsigned lds_addr = uni(static_cast<unsigned>(
+      reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
+
+  auto issue_one = [&](int ks, int q) {
+    const unsigned st = lds_addr + (ks & (STAGES - 1)) * TALL_STAGE_BYTES;
+    if (q < LQ) {
+      load_to_lds(rows.woff[q], rows.wbase[q] + static_cast<size_t>(ks) * rows.wkstride,
+                  st + (wave * LQ + q) * 1024);
+    } else {
+      load_to_lds(rows.toff[q - LQ], rows.tbase + static_cast<size_t>(ks) * rows.tkstride,
+                  st + TN * TK * 2 + (wave + 8 * (q - LQ)) * 1024);
+    }
+  };
+  auto issue = [&](int ks) {
+#pragma unroll
+    for (int q = 0; q < NLD; ++q) issue_one(ks, q);
+  };
+
+  const int swz = (r32 >> 2) & 3;
+  const int rd0 = r32 * 64 + ((kq ^ swz) << 4);
+  const int rd1 = r32 * 64 + (((kq ^ swz) ^ 2) << 4);
+  const int pk0 = (r32 >> 4) * 1024 + ((kq * 16 + (r32 & 15)) << 4);
+  const int pk1 = (r32 >> 4) * 1024 + (((2 + kq) * 16 + (r32 & 15)) << 4);
+  const int ra0 = rows.wpacked ? pk0 : rd0, ra1 = rows.wpacked ? pk1 : rd1;
+  const int rb0 = rows.tpacked ? pk0 : rd0, rb1 = rows.tpacked ? pk1 : rd1;
+  auto read_a = [&](TallFrags& f, int ks, int kk, int i) {
+    const unsigned char* st = lds + (ks & (STAGES - 1)) * TALL_STAGE_BYTES + (kk == 0 ? ra0 : ra1);
+    f.a[i] = *reinterpret_cast<const uint4*>(st + wblk[i] * 64);
+  };
+  auto read_b = [&](TallFrags& f, int ks, int kk, int j) {
+    const unsigned char* st = lds + (ks & (STAGES - 1)) * TALL_STAGE_BYTES + (kk == 0 ? rb0 : rb1);
+    if (j < NTB) f.b[j] = *reinterpret_cast<const uint4*>(st + TN * TK * 2 + (tok0 + j * 32) * 64);
+  };
+  auto read = [&](TallFrags& f, int ks, int kk) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) read_a(f, ks, kk, i);
+#pragma unroll
+    for (int j = 0; j < 5; ++j) read_b(f, ks, kk, j);
+  };
+  auto mfma_block = [&](const TallFrags& f, int j) {
+    if (j < NTB) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) acc[i][j] = mma32(f.a[i], f.b[j], acc[i][j]);
+    }
+  };
+
+  TallFrags f0, f1;
+  auto step = [&](int ks, auto pending_tag, auto refill_tag, auto last_tag) {
+    constexpr int PENDING = decltype(pending_tag)::value;
+    constexpr int REFILL = decltype(refill_tag)::value;
+    constexpr bool LAST = decltype(last_tag)::value;
+    read(f1, ks, 1);
+#pragma unroll
+    for (int j = 0; j < 5; ++j) mfma_block(f0, j);
+#pragma unroll
+    for (int n = 0; n < 2 + NTB; ++n) {  // the reads spread between the matrix instructions
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (!LAST) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // nobody still reads stage ks after the barrier
+      wait_vm<PENDING>();
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int g = 0; g < 5; ++g) {
+        mfma_block(f1, g);
+        __builtin_amdgcn_sched_barrier(0);
+        if (REFILL == 1 && g < NLD) issue_one(ks + STAGES, g);
+        if (g < 2) read_a(f0, ks + 1, 0, g);
+        read_b(f0, ks + 1, 0, g);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 5; ++j) mfma_block(f1, j);
+    }
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, NLD>;
+  using I2 = std::integral_constant<int, 2 * NLD>;
+  using R0 = std::integral_constant<int, 0>;
+  using R1 = std::integral_constant<int, 1>;
+#pragma unroll
+  for (int st = 0; st < STAGES; ++st) issue(st);
+  wait_vm<3 * NLD>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  read(f0, 0, 0);
+  int ks = 0;
+  for (; ks + STAGES < ksteps; ++ks) step(ks, I2{}, R1{}, std::false_type{});
+  step(ks++, I2{}, R0{}, std::false_type{});
+  step(ks++, I1{}, R0{}, std::false_type{});
+  step(ks++, I0{}, R0{}, std::false_type{});
+  step(ks, I0{}, R0{}, std::true_type{});
+  __syncthreads();  // the stages are free for the epilogue
+}
+
+// dispatch on the wave's position: waves 0..3 own token rows 0..159 (all five blocks live, three
+// token loads), waves 4..7 rows 160..319 (four or five blocks, two loads)
+__device__ __forceinline__ void tall_gemm_dispatch(const TallRows& rows, int ksteps, const int (&wblk)[2],
+                                                   int tok0, int ntb, f32x16 (&acc)[2][5]) {
+  if (uni(static_cast<int>(threadIdx.x >> 6)) < 4) {
+    tall_gemm<5, 3>(rows, ksteps, wblk, tok0, acc);
+  } else if (ntb > 4) {
+    tall_gemm<5, 2>(rows, ksteps, wblk, tok0, acc);
+  } else {
+    tall_gemm<4, 2>(rows, ksteps, wblk, tok0, acc);
+  }
+}
+
+// the 16-row token block L (0..19) this wave loads as its q-th token load, or -1
+__device__ __forceinline__ int tall_token_block(int q) {
+  const int L = static_cast<int>(threadIdx.x >> 6) + 8 * q;
+  return L < TALL_TM / 16 ? L : -1;
+}
+
+__device__ __noinline__ void tall_gateup_task(const Params& p, const TileDesc& tile_in, int m, int nblk) {
+  const int H = uni(p.H), I = uni(p.I), K = uni(p.K);
+  TileDesc tile;
+  tile.expert = uni(tile_in.expert);
+  tile.row0 = uni(tile_in.row0);
+  tile.rows = uni(tile_in.rows);
+  const int n0 = uni(nblk) * G1_COLS;
+  const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const unsigned short* w13 = uni(reinterpret_cast<const unsigned short*>(p.ffn1)) +
+                              static_cast<size_t>(tile.expert) * 2 * I * H;
+  TallRows rows;
+  rows.wpacked = uni(p.ffn1_packed != nullptr ? 1 : 0) != 0;
+  rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
+  rows.tkstride = static_cast<unsigned>(TK * 2);
+  rows.tpacked = false;
+  rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
+#pragma unroll
+  for (int q = 0; q < LQ; ++q) {
+    const int row = stage_row(q);
+    if (rows.wpacked) {
+      const int B = wave * LQ + q;
+      const int half = B >> 3, b8 = B & 7;
+      const size_t task = static_cast<size_t>(tile.expert) * (I / 32) + (n0 / 32 + (b8 >> 1));
+      rows.wbase[q] = uni(reinterpret_cast<const unsigned char*>(p.ffn1_packed)) +
+                      task * (static_cast<size_t>(H / 32) * 4096) + (2 * half + (b8 & 1)) * 1024;
+      rows.woff[q] = lane * 16;
+    } else {
+      const int wrow = row < G1_COLS ? n0 + row : I + n0 + (row - G1_COLS);
+      rows.wbase[q] = reinterpret_cast<const unsigned char*>(w13);
+      rows.woff[q] = static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 3; ++q) {
+    const int L = max(tall_token_block(q), 0);
+    const int row = L * 16 + (lane >> 2);
+    const int tok = ldc(&p.perm[tile.row0 + min(row, tile.rows - 1)]) / K;
+    rows.toff[q] = static_cast<unsigned>(tok) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+  }
+  const int wn = wave & 3, wm = wave >> 2;
+  const int wblk[2] = {wn * 32, G1_COLS + wn * 32};  // 32 gate rows and the matching 32 up rows
+  const int tok0 = wm * 160;
+  const int ntb = uni(min(5, (tile.rows - tok0 + 31) / 32));
+  // this wave's 32 columns are k-step (n0 + 32*wn)/32 of the tile's h
+  unsigned char* h = uni(reinterpret_cast<unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I) +
+                     static_cast<size_t>((n0 + wn * 32) / 32) * (HT_ROWS * 64);
+  f32x16 acc[2][5];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 5; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  tall_gemm_dispatch(rows, H / TK, wblk, tok0, ntb, acc);
+
+  const int r32 = lane & 31, kq = lane >> 5;
+  constexpr int SLD = 32 + 8;  // slab row stride, bf16 elements
+  unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * 32 * SLD;
+#pragma unroll
+  for (int j = 0; j < 5; ++j) {
+    if (j < ntb) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        float hv[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) hv[v] = silu_mul_fast(acc[0][j][g4 * 4 + v], acc[1][j][g4 * 4 + v]);
+        uint2 pk;
+        pk.x = pack_bf16(hv[0], hv[1]);
+        pk.y = pack_bf16(hv[2], hv[3]);
+        *reinterpret_cast<uint2*>(slab + r32 * SLD + g4 * 8 + kq * 4) = pk;
+      }
+      lds_wave_sync();
+#pragma unroll
+      for (int b16 = 0; b16 < 2; ++b16) {
+        // one 1 KiB run: 16-row block b16 of this token block, chunk lane / 16 of row lane % 16
+        const int rr = b16 * 16 + (lane & 15), cc = (lane >> 4) * 8;
+        const int trow = tok0 + j * 32 + rr;
+        const uint4 v = *reinterpret_cast<const uint4*>(slab + rr * SLD + cc);
+        if (trow < tile.rows) st16_through(h + ((tok0 + j * 32) / 16 + b16) * 1024 + lane * 16, v);
+      }
+      lds_wave_sync();
+    }
+  }
+}
+
+__device__ __noinline__ void tall_down_task(const Params& p, const TileDesc& tile_in, int m, int nblk) {
+  const int H = uni(p.H), I = uni(p.I);
+  TileDesc tile;
+  tile.expert = uni(tile_in.expert);
+  tile.row0 = uni(tile_in.row0);
+  tile.rows = uni(tile_in.rows);
+  const int n0 = uni(nblk) * TN;
+  const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const unsigned short* w2 = uni(reinterpret_cast<const unsigned short*>(p.ffn2)) +
+                             static_cast<size_t>(tile.expert) * H * I;
+  TallRows rows;
+  rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I);
+  rows.tkstride = static_cast<unsigned>(HT_ROWS * 64);
+  rows.tpacked = true;
+  rows.wpacked = uni(p.ffn2_packed != nullptr ? 1 : 0) != 0;
+  rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
+#pragma unroll
+  for (int q = 0; q < LQ; ++q) {
+    const int row = stage_row(q);
+    if (rows.wpacked) {
+      const int B = wave * LQ + q;
+      const size_t task = static_cast<size_t>(tile.expert) * (H / 64) + (n0 / 64 + (B >> 2));
+      rows.wbase[q] = uni(reinterpret_cast<const unsigned char*>(p.ffn2_packed)) +
+                      task * (static_cast<size_t>(I / 32) * 4096) + (B & 3) * 1024;
+      rows.woff[q] = lane * 16;
+    } else {
+      rows.wbase[q] = reinterpret_cast<const unsigned char*>(w2);
+      rows.woff[q] = static_cast<unsigned>(n0 + row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 3; ++q) rows.toff[q] = static_cast<unsigned>(max(tall_token_block(q), 0) * 1024 + lane * 16);
+  const int wn = wave & 3, wm = wave >> 2;
+  const int wblk[2] = {wn * 64, wn * 64 + 32};
+  const int tok0 = wm * 160;
+  const int ntb = uni(min(5, (tile.rows - tok0 + 31) / 32));
+  const int r32 = lane & 31, kq = lane >> 5;
+  unsigned short* y = uni(reinterpret_cast<unsigned short*>(p.y)) + n0 + wn * 64 + (lane & 7) * 8;
+  float roww[5];
+  int dstrow[5];
+  {
+    const float* row_w = uni(p.row_w) + tile.row0;
+    const int* perm = uni(p.perm) + tile.row0;
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+      const int myrow = tok0 + j * 32 + r32;
+      const bool valid = myrow < tile.rows;
+      roww[j] = valid ? ldc(&row_w[myrow]) : 0.0f;
+      dstrow[j] = valid ? ldc(&perm[myrow]) : -1;
+    }
+  }
+  f32x16 acc[2][5];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 5; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  tall_gemm_dispatch(rows, I / TK, wblk, tok0, ntb, acc);
+
+  constexpr int SLD = 64 + 8;  // slab row stride, bf16 elements
+  unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * (32 * SLD);
+#pragma unroll
+  for (int j = 0; j < 5; ++j) {
+    if (j < ntb) {
+      const float w = roww[j];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          uint2 pk;
+          pk.x = pack_bf16(acc[i][j][g4 * 4 + 0] * w, acc[i][j][g4 * 4 + 1] * w);
+          pk.y = pack_bf16(acc[i][j][g4 * 4 + 2] * w, acc[i][j][g4 * 4 + 3] * w);
+          *reinterpret_cast<uint2*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) = pk;
+        }
+      lds_wave_sync();
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        // eight lanes store one row's 128 bytes: rows 8*it .. 8*it+7
+        const int q = lane >> 3;
+        int dst = -1;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          const int d = __builtin_amdgcn_readlane(dstrow[j], it * 8 + r);
+          dst = q == r ? d : dst;
+        }
+        const uint4 v = *reinterpret_cast<const uint4*>(slab + (it * 8 + q) * SLD + (lane & 7) * 8);
+        if (dst >= 0) st16_through(y + static_cast<size_t>(dst) * H, v);
+      }
+      lds_wave_sync();
+    }
+  }
+}
+
 
 // combine: out[t] = sum over slots, in slot order, of y[t*K+slot]
 // (refFullMoe.h:35,62-65).
@@ -1143,7 +1483,11 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
         const unsigned m = lo + j / nt1;
         if (p.trace) t_ready = wall_clock64();
         const TileDesc tile = ld_tile(&p.mtiles[m]);
-        tiled_gateup_task(p, tile, static_cast<int>(m), static_cast<int>(j % nt1));
+        if (tile.rows > TM) {
+          tall_gateup_task(p, tile, static_cast<int>(m), static_cast<int>(j % nt1));
+        } else {
+          tiled_gateup_task(p, tile, static_cast<int>(m), static_cast<int>(j % nt1));
+        }
         wg_arrive<false>(&p.g1_done[m].v, &sh);
         trace(t_dyn0 + lo * nt1 + j, 3, m, t_fetch, t_ready);
       } else {
@@ -1153,7 +1497,11 @@ __global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
         if (ok) {
           if (p.trace) t_ready = wall_clock64();
           const TileDesc tile = ld_tile(&p.mtiles[m]);
-          tiled_down_task(p, tile, static_cast<int>(m), static_cast<int>(jj % nt2));
+          if (tile.rows > TM) {
+            tall_down_task(p, tile, static_cast<int>(m), static_cast<int>(jj % nt2));
+          } else {
+            tiled_down_task(p, tile, static_cast<int>(m), static_cast<int>(jj % nt2));
+          }
           if (wg_arrive<false>(&ctl->g2_done.v, &sh) == n2_total - 1u) wg_broadcast_flag(p, FLAG_G2);
           trace(t_dyn0 + nm * nt1 + lo * nt2 + jj, 4, m, t_fetch, t_ready);
         }

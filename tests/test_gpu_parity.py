@@ -115,6 +115,8 @@ def test_relaunch_and_smaller_batch():
     (700, 512, 4, 2, 256),      # several 256-row tiles per expert, ragged tail
     (64, 256, 200, 6, 128),     # E > 128: two expert slabs in the router; tiny tiles
     (1, 256, 8, 2, 128),        # a single token
+    (1100, 256, 8, 2, 128),     # ~275 rows per expert: tall tiles (a tail of <= 64 rows joins the full tile)
+    (1180, 512, 4, 1, 256),     # ~295 rows per expert, top-1; some experts beyond 320 rows (tile + tail tile)
 ])
 def test_tiled_variant_forced(shape):
     T, H, E, k, I = shape
