@@ -516,20 +516,25 @@ __device__ __noinline__ void tiled_scan_task(const Params& p) {
       const int c = e < r.E ? ldc(&r.expert_count[e]) : 0;
       const int incl = wave_inclusive_scan(c);
       const int off = base + incl - c;
-      // a tail of at most TALL_EXTRA rows joins the last full tile (a tall tile)
-      const bool tall = c > TM && (c % TM) != 0 && (c % TM) <= TALL_EXTRA;
-      const int nt = tall ? c / TM : (c + TM - 1) / TM;
+      // Tiles of up to TALL_TM rows where that saves passes over the expert's weights
+      // (a tall tile costs about an eighth more than one of TM rows): tiles keep TM
+      // rows as long as the rest still fits the remaining tiles at TALL_TM each.
+      const int nt_norm = (c + TM - 1) / TM, nt_tall = (c + TALL_TM - 1) / TALL_TM;
+      const int nt = nt_tall * 9 < nt_norm * 8 ? nt_tall : nt_norm;
       const int tincl = wave_inclusive_scan(nt);
       const int toff = tile_base + tincl - nt;
       if (e < r.E) {
         stc(&r.expert_offset[e], off);
+        int done = 0;
         for (int i = 0; i < nt; ++i) {
+          const int left = c - done;
+          const int tr = max(min(TM, left), left - TALL_TM * (nt - 1 - i));
           if (toff + i < r.max_mtiles) {
-            const int tr = (tall && i == nt - 1) ? c - i * TM : min(TM, c - i * TM);
             stc16(&r.mtiles[toff + i],
-                  make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + i * TM),
+                  make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + done),
                              static_cast<unsigned>(tr), 0u));
           }
+          done += tr;
         }
       }
       base += __shfl(incl, 63, 64);
