@@ -33,6 +33,17 @@ struct BF16 {
 // polls the counter and then loads. Inputs (tokens, weights) are never written
 // while the kernel runs and use ordinary cached loads.
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+// The launch parameters where the dispatch put them: the kernels take one
+// argument, a Params by value, which starts the kernel-argument segment.
+#if defined(FMOE_PARAMS_IN_KERNARG)
+__device__ __forceinline__ ParamsRef kernel_params() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return *(const __attribute__((address_space(4))) Params*)__builtin_amdgcn_kernarg_segment_ptr();
+#else
+  return *static_cast<const Params*>(nullptr);
+#endif
+}
+#endif
 
 // Every pointer in Params is HBM: saying so lets the compiler emit global_*
 // instead of flat_* memory instructions (flat ones also count as LDS traffic).
@@ -137,7 +148,7 @@ __device__ __forceinline__ unsigned wave_arrive(unsigned* counter) {
 
 // Called by the worker that completed a phase (after wave_arrive told it so, or
 // after its own release fence): raises the phase flag of every workgroup.
-__device__ __forceinline__ void broadcast_flag(const Params& p, int which) {
+__device__ __forceinline__ void broadcast_flag(ParamsRef p, int which) {
   const int n = p.n_groups;
   WgFlags* flags = p.wgflags;
   for (int g = lane_id(); g < n; g += 64) st_relaxed(&flags[g].f[which], 1u);
@@ -183,6 +194,18 @@ __device__ __forceinline__ T* uniform_ptr(T* ptr) {
   const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
   const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
   return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
+// The launch parameters as a function that is not inlined receives them: arguments
+// arrive in vector registers, and only a pointer known to be uniform gets scalar loads.
+__device__ __forceinline__ ParamsRef uniform_params(ParamsRef p) {
+#if defined(__HIP_DEVICE_COMPILE__) && defined(FMOE_PARAMS_IN_KERNARG)
+  const unsigned long long v = (unsigned long long)&p;
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
+  return *(const __attribute__((address_space(4))) Params*)((static_cast<unsigned long long>(hi) << 32) | lo);
+#else
+  return p;
+#endif
 }
 // 16 bytes read at agent scope (one instruction; an atomic load carries 8 at
 // most): the load bypasses whatever this XCD's L2 holds for the line, so it sees
@@ -340,7 +363,7 @@ __device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
 // first of equal values because it compares with a strict '>'). val[j] is
 // ordered_bits of expert lane + 64*j. lex: MAX_TOPK doubles of LDS private to
 // the wave.
-__device__ __forceinline__ void router_select_max(const Params& p, int t,
+__device__ __forceinline__ void router_select_max(ParamsRef p, int t,
                                                   unsigned (&val)[MAX_EXPERTS / 64], double* lex) {
   constexpr int MAXEPL = MAX_EXPERTS / 64;
   const int lane = lane_id();
@@ -407,7 +430,7 @@ struct RouteTables {
   float* row_w;
   TileDesc* mtiles;
 };
-__device__ __forceinline__ RouteTables route_tables(const Params& p) {
+__device__ __forceinline__ RouteTables route_tables(ParamsRef p) {
   RouteTables r;
   r.T = p.T;
   r.E = p.E;

@@ -183,7 +183,15 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   // workgroups at most, to leave workers for the weights).
   const int dot_tasks = ((T + fmoe::ROUTER_TOK - 1) / fmoe::ROUTER_TOK) *
                         ((d.experts + fmoe::ROUTER_EXP - 1) / fmoe::ROUTER_EXP);
-  const int routing_groups = std::max((dot_tasks + 3) / 4, (T + 4) / 4);
+  // bf16 layers run the logit chains on the matrix core, 16 tokens x 16 experts
+  // per workgroup, while every such task finds a workgroup of its own
+  const int dot16_tasks = ((T + 15) / 16) * ((d.experts + 15) / 16);
+  p.dot16 = (d.dtype == FLASH_MOE_BF16 && d.hidden % fmoe::DOT16_KC == 0 &&
+             dot16_tasks <= p.n_groups)
+                ? 1
+                : 0;
+  const int routing_groups =
+      std::max(p.dot16 ? dot16_tasks : (dot_tasks + 3) / 4, (T + 4) / 4);
   // Early mode hands out the tasks of every expert, used or not (an unused one
   // costs a ticket and a wasted first round of loads), so it needs a batch that
   // reaches most experts: T*k >= E (measured on the 30B shape, with it / without:

@@ -30,6 +30,7 @@ constexpr int G2_NB = FMOE_G2_NB;  // 16-wide column blocks per down wave task
 constexpr int COMBINE_COLS = 256;
 constexpr int ROUTER_TOK = 8;    // streaming variant: tokens per router dot task
 constexpr int ROUTER_EXP = 8;    // streaming variant: experts per router dot task
+constexpr int DOT16_KC = 256;    // streaming variant, matrix-core router: k per LDS stage
 constexpr int SCAN_LDS_WORDS = 1024;  // mask words (experts x 64-token words) the small-batch scan keeps in LDS
 constexpr int EARLY_MAX_TOKENS = 64;   // batches up to this size take their gate/up weights before the routing is known
 constexpr int MAX_EXPERTS = 256;  // experts are spread 64 per wave register slot
@@ -126,8 +127,24 @@ struct Params {
   int early;                       // 1: row tile e belongs to expert e (empty or not), so gate/up tasks are
                                    //    handed out at launch and fetch their first weights under the routing
   int tpad;                        // dense mode: h rows reserved per expert
+  int dot16;                       // 1 (streaming variant, bf16): the logit chains run on the matrix core, 16 tokens x
+                                   //    16 experts per workgroup, on the first workgroups before they take tickets
   TraceRec* trace;    // null unless tracing; indexed by ticket
   unsigned trace_cap;
 };
+
+// How device code reaches the launch parameters. A kernel parameter whose address
+// is passed to a function is copied to the wave's private memory first, and every
+// field read in a task then goes through the vector memory pipeline, behind the
+// weight loads. A kernel that defines FMOE_PARAMS_IN_KERNARG before including
+// this header reads them in place in the kernel-argument segment instead
+// (constant address space): a field costs a scalar load that the scalar cache
+// serves. That is what short tasks want (the streaming variant); the tiled
+// variant's GEMM tasks have no register to spare for it and keep the copy.
+#if defined(__HIP_DEVICE_COMPILE__) && defined(FMOE_PARAMS_IN_KERNARG)
+typedef const __attribute__((address_space(4))) Params& ParamsRef;
+#else
+typedef const Params& ParamsRef;
+#endif
 
 }  // namespace fmoe

@@ -27,6 +27,7 @@
 // Replaces, for this regime, the reference's moeKernel
 // (src/hip/kernel/moeKernel.h:37-107), its task executors
 // (src/hip/kernel/tasks/*.h) and its queue (src/hip/taskSystem/*.h).
+#define FMOE_PARAMS_IN_KERNARG 1
 #include "moe_device.h"
 
 namespace fmoe {
@@ -53,7 +54,8 @@ constexpr int ROUTER_LDS_FLOATS = 2 * ROUTER_EXP * ROUTER_LD;  // per wave
 extern __shared__ __align__(16) float lds_dyn[];  // ROUTER_LDS_FLOATS per wave
 
 template <typename DT>
-__device__ __noinline__ void router_dot_task(const Params& p, int tg, int eg) {
+__device__ __noinline__ void router_dot_task(ParamsRef pv, int tg, int eg) {
+  ParamsRef p = uniform_params(pv);
   typedef typename DT::elem elem;
   constexpr int EPV = DT::EPV;
   constexpr int CH_ROW = ROUTER_KC / EPV;               // 16-byte chunks per staged row
@@ -185,8 +187,142 @@ __device__ __noinline__ void router_dot_task(const Params& p, int tg, int eg) {
   if (ei == 0 && t < T) add_relaxed(&p.tok_arrive[t], 1u);
 }
 
+// The same chains on the matrix core, for bf16 layers: V_MFMA_F32_16X16X4_F32 adds
+// its four products to the accumulator one after the other in k order, one
+// rounding each, so a chain of them is the same sequential sum (and a dependent
+// chain issues back to back, 32 cycles an instruction: 512 of them for H = 2048
+// against 2048 dependent FMAs on the vector unit). A whole workgroup takes 16
+// tokens x 16 experts: wave 0 only multiplies, waves 1..4 prepare its operands so
+// that it has nothing else to do: they load 32 bytes of a row (16 k), widen them
+// to float and leave them in LDS in the order the instruction wants them: the 16
+// k of a group as [k % 4][row][k / 4], so lane l of the multiplying wave (row
+// l % 16, k % 4 = l / 16) reads its operand of four consecutive instructions with
+// one 16-byte read at 16 * l. Two stages of DOT16_KC k; one workgroup barrier per
+// stage; the preparing waves hold the loads of eight stages in registers.
+// Called by all eight waves of the workgroup.
+constexpr int DOT16_GROUPS = DOT16_KC / 16;             // 16-k groups per stage
+constexpr int DOT16_OP_BYTES = DOT16_GROUPS * 1024;     // one operand of one stage
+constexpr int DOT16_STAGE_BYTES = 2 * DOT16_OP_BYTES;   // expert rows, then token rows
+constexpr int DOT16_AHEAD = 8;                          // stages whose loads are in flight together (even)
+
+__device__ __noinline__ void router_dot16_task(ParamsRef pv, int tg, int eg) {
+  ParamsRef p = uniform_params(pv);
+  const int H = p.H, E = p.E, T = p.T;
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int nc = H / DOT16_KC;
+  unsigned char* lds = reinterpret_cast<unsigned char*>(lds_dyn);
+  auto barrier = [] {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  if (wave == 0) {
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    const unsigned char* mine = lds + lane * 16;
+    float4 wc, xc, wn, xn;
+    barrier();  // stage 0 is written
+    wc = *reinterpret_cast<const float4*>(mine);
+    xc = *reinterpret_cast<const float4*>(mine + DOT16_OP_BYTES);
+    for (int c = 0; c < nc; ++c) {
+      const unsigned char* st = mine + (c & 1) * DOT16_STAGE_BYTES;
+      const unsigned char* st_next = mine + ((c + 1) & 1) * DOT16_STAGE_BYTES;
+#pragma unroll
+      for (int g = 0; g < DOT16_GROUPS; ++g) {
+        if (g + 1 < DOT16_GROUPS) {
+          wn = *reinterpret_cast<const float4*>(st + (g + 1) * 1024);
+          xn = *reinterpret_cast<const float4*>(st + DOT16_OP_BYTES + (g + 1) * 1024);
+        } else {
+          // every read of this stage has returned: the stage may be refilled, and
+          // the next one is complete once the others have arrived too
+          barrier();
+          if (c + 1 < nc) {
+            wn = *reinterpret_cast<const float4*>(st_next);
+            xn = *reinterpret_cast<const float4*>(st_next + DOT16_OP_BYTES);
+          }
+        }
+        // the reads of the next group go out before this group's instructions, not after
+        __builtin_amdgcn_sched_barrier(0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wc.x, xc.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wc.y, xc.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wc.z, xc.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wc.w, xc.w, acc, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        wc = wn;
+        xc = xn;
+      }
+    }
+    // acc[v] of lane l: expert 16*eg + 4*(l/16) + v, token 16*tg + l%16
+    const int t = tg * 16 + (lane & 15);
+    const int e0 = eg * 16 + 4 * (lane >> 4);
+    if (t < T) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int e = e0 + v;
+        if (e < E) {
+          float x = acc[v];
+          if (p.bias != nullptr) x = __fadd_rn(x, as_global(p.bias)[e]);
+          stc(&p.cand[static_cast<size_t>(t) * E + e], make_key(x, e, true));
+        }
+      }
+    }
+    fence_release();
+    if (lane < 16 && t < T) add_relaxed(&p.tok_arrive[t], 1u);
+  } else if (wave <= 4) {
+    // lane -> (row, group): four lanes cover 128 contiguous bytes of a row
+    const int hl = (wave - 1) * 64 + lane;
+    const int row = (hl & 63) >> 2;
+    const int g = (hl >> 6) * 4 + (hl & 3);
+    const unsigned short* wsrc = reinterpret_cast<const unsigned short*>(p.gate) +
+                                 static_cast<size_t>(min(eg * 16 + row, E - 1)) * H + g * 16;
+    const unsigned short* xsrc = reinterpret_cast<const unsigned short*>(p.tokens) +
+                                 static_cast<size_t>(min(tg * 16 + row, T - 1)) * H + g * 16;
+    unsigned char* dst = lds + g * 1024 + row * 16;
+    struct Regs {
+      uint4 w0, w1, x0, x1;
+    };
+    auto load = [&](Regs& r, int c) {
+      const int k = min(c, nc - 1) * DOT16_KC;  // past the end: the last stage again, never written
+      r.w0 = ld16(wsrc + k);
+      r.w1 = ld16(wsrc + k + 8);
+      r.x0 = ld16(xsrc + k);
+      r.x1 = ld16(xsrc + k + 8);
+    };
+    auto widen = [](unsigned char* d, const uint4& a, const uint4& b) {
+      // k % 4 = 0 and 1: low and high halves of the even words; 2 and 3: of the odd words
+      *reinterpret_cast<uint4*>(d) = make_uint4(a.x << 16, a.z << 16, b.x << 16, b.z << 16);
+      *reinterpret_cast<uint4*>(d + 256) =
+          make_uint4(a.x & 0xFFFF0000u, a.z & 0xFFFF0000u, b.x & 0xFFFF0000u, b.z & 0xFFFF0000u);
+      *reinterpret_cast<uint4*>(d + 512) = make_uint4(a.y << 16, a.w << 16, b.y << 16, b.w << 16);
+      *reinterpret_cast<uint4*>(d + 768) =
+          make_uint4(a.y & 0xFFFF0000u, a.w & 0xFFFF0000u, b.y & 0xFFFF0000u, b.w & 0xFFFF0000u);
+    };
+    // The loads of DOT16_AHEAD stages go out together (straight-line code, so each
+    // stage waits for exactly its own four): a load takes 2 to 3 us to come back
+    // here, three times what the multiplying wave spends on a stage.
+    for (int c0 = 0; c0 < nc; c0 += DOT16_AHEAD) {
+      Regs r[DOT16_AHEAD];
+#pragma unroll
+      for (int i = 0; i < DOT16_AHEAD; ++i) load(r[i], c0 + i);
+#pragma unroll
+      for (int i = 0; i < DOT16_AHEAD; ++i) {
+        if (c0 + i < nc) {
+          unsigned char* d = dst + (i & 1) * DOT16_STAGE_BYTES;
+          widen(d, r[i].w0, r[i].w1);
+          widen(d + DOT16_OP_BYTES, r[i].x0, r[i].x1);
+          barrier();  // the stage is written; the multiplying wave is done with the one before
+        }
+      }
+    }
+    barrier();  // the multiplying wave has read everything: the LDS is free again
+  } else {
+    for (int c = 0; c <= nc; ++c) barrier();
+  }
+}
+
 // All expert groups of token t have left their keys: pick the winners.
-__device__ __noinline__ void router_select_task(const Params& p, int t) {
+__device__ __noinline__ void router_select_task(ParamsRef pv, int t) {
+  ParamsRef p = uniform_params(pv);
   constexpr int MAXEPL = MAX_EXPERTS / 64;
   const int lane = lane_id();
   unsigned val[MAXEPL];  // the ordered logit bits are the upper half of a candidate key
@@ -209,7 +345,8 @@ __device__ __noinline__ void router_select_task(const Params& p, int t) {
 // permutation stage (it runs one GEMV per (token, slot)); this is the
 // token-grouping the streaming and tiled GEMMs need. For small batches the same
 // wave also writes the permutation.
-__device__ __noinline__ void scan_task(const Params& p) {
+__device__ __noinline__ void scan_task(ParamsRef pv) {
+  ParamsRef p = uniform_params(pv);
   const RouteTables r = route_tables(p);
   const int fuse = p.fuse_scatter;
   Control* ctl = p.ctl;
@@ -304,7 +441,8 @@ __device__ __noinline__ void scan_task(const Params& p) {
 // loads of masks and routing at the start, the stores at the end.
 static_assert(SCAN_LDS_WORDS * 12 + MAX_EXPERTS * 4 <= ROUTER_LDS_FLOATS * 4, "scan tables exceed the wave's LDS");
 
-__device__ __noinline__ void scan_scatter_small_task(const Params& p) {
+__device__ __noinline__ void scan_scatter_small_task(ParamsRef pv) {
+  ParamsRef p = uniform_params(pv);
   const RouteTables r = route_tables(p);
   Control* ctl = p.ctl;
   const int lane = lane_id();
@@ -403,7 +541,7 @@ __device__ __noinline__ void scan_scatter_small_task(const Params& p) {
   lds_wave_sync();
 }
 
-__device__ void scatter_task(const Params& p, int t) {
+__device__ void scatter_task(ParamsRef p, int t) {
   const RouteTables r = route_tables(p);
   const int lane = lane_id();
   if (lane < r.K) scatter_entry(r, t * r.K + lane);
@@ -414,7 +552,7 @@ __device__ void scatter_task(const Params& p, int t) {
 // Wave-uniform bounded wait for this workgroup's copy of a phase flag. Only one
 // wave of the workgroup polls HBM; the others watch a word in LDS that the
 // polling wave sets (1 = flag seen, 2 = failed).
-__device__ __forceinline__ bool wait_flag(const Params& p, int which, unsigned* lds_flag,
+__device__ __forceinline__ bool wait_flag(ParamsRef p, int which, unsigned* lds_flag,
                                           unsigned* lds_poller) {
   int ok = 1;
   if (lane_id() == 0) {
@@ -558,7 +696,7 @@ struct RoundSteps {
 // permutation gives them), and its first row is the number of entries that name
 // a lower expert. Lanes 0..15 (and their copies in the other lane groups) get
 // the entry of row min(lane & 15, rows - 1). For batches of at most 64 tokens.
-__device__ __forceinline__ void tile_from_topk(const Params& p, int e, int& row0, int& rows,
+__device__ __forceinline__ void tile_from_topk(ParamsRef p, int e, int& row0, int& rows,
                                                int& entry) {
   const int lane = lane_id();
   const int r16 = lane & 15;
@@ -600,7 +738,7 @@ __device__ __forceinline__ void tile_from_topk(const Params& p, int e, int& row0
 // the tile has more than 16*RB rows, nothing was written, and the caller runs
 // the task again from the tile table with more row blocks.
 template <typename DT, int RB, bool DENSE, bool EARLY>
-__device__ __forceinline__ int gateup_body(const Params& p, TileDesc& tile, int nblk,
+__device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk,
                                            unsigned* lds_flag, unsigned* lds_poller) {
   typedef typename DT::elem elem;
   constexpr int EPV = DT::EPV;
@@ -693,16 +831,25 @@ __device__ __forceinline__ int gateup_body(const Params& p, TileDesc& tile, int 
 }
 
 template <typename DT, int RB, bool DENSE>
-__device__ __noinline__ void gateup_task(const Params& p, const TileDesc& tile_in, int nblk) {
-  TileDesc tile = tile_in;
+__device__ __noinline__ void gateup_task(ParamsRef pv, int expert, int row0, int rows, int nblk) {
+  // (the row tile arrives as three integers: a struct by value makes the callee save
+  // and restore every callee-saved register it touches, a struct by reference costs
+  // a trip to the caller's private memory)
+  ParamsRef p = uniform_params(pv);
+  TileDesc tile;
+  tile.expert = expert;
+  tile.row0 = row0;
+  tile.rows = rows;
+  tile.pad = 0;
   gateup_body<DT, RB, DENSE, false>(p, tile, nblk, nullptr, nullptr);
 }
 
 // tile.expert is set on entry; the rest of the descriptor is filled in once the
 // routing is known
 template <typename DT>
-__device__ __noinline__ int gateup_early_task(const Params& p, TileDesc& tile, int nblk,
+__device__ __noinline__ int gateup_early_task(ParamsRef pv, TileDesc& tile, int nblk,
                                               unsigned* lds_flag, unsigned* lds_poller) {
+  ParamsRef p = uniform_params(pv);
   return gateup_body<DT, 1, false, true>(p, tile, nblk, lds_flag, lds_poller);
 }
 
@@ -713,8 +860,14 @@ __device__ __noinline__ int gateup_early_task(const Params& p, TileDesc& tile, i
 // on h, so their first loads are issued before the wait for the tile's
 // gate/up tasks. Returns false if that wait failed.
 template <typename DT, int RB, bool DENSE>
-__device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, int nblk, unsigned* dep,
-                          unsigned dep_target) {
+__device__ __noinline__ bool down_task(ParamsRef pv, int expert, int row0, int rows, int nblk,
+                                       unsigned* dep, unsigned dep_target) {
+  ParamsRef p = uniform_params(pv);
+  TileDesc tile;
+  tile.expert = expert;
+  tile.row0 = row0;
+  tile.rows = rows;
+  tile.pad = 0;
   typedef typename DT::elem elem;
   constexpr int EPV = DT::EPV;
   constexpr int NA = G2_NB;
@@ -801,7 +954,7 @@ __device__ __noinline__ bool down_task(const Params& p, const TileDesc& tile, in
 // out[t, c0..c0+256) = sum over slots, in slot order, of the weighted rows
 // (refFullMoe.h:35,62-65; src/hip/kernel/tasks/internal/reduceBlock.h:35-53).
 template <typename DT>
-__device__ void combine_task(const Params& p, int t, int chunk) {
+__device__ void combine_task(ParamsRef p, int t, int chunk) {
   const int lane = lane_id();
   const int c = chunk * COMBINE_COLS + lane * 4;
   if (c < p.H) {
@@ -847,9 +1000,10 @@ __device__ void combine_task(const Params& p, int t, int chunk) {
 // The combine items slot, slot + n_workers, ... of one worker (a function of its
 // own so that the worker loop's registers are not shared with it).
 template <typename DT>
-__device__ __noinline__ void combine_items(const Params& p, unsigned slot, unsigned nc,
+__device__ __noinline__ void combine_items(ParamsRef pv, unsigned slot, unsigned nc,
                                            unsigned ncomb, unsigned worker, unsigned id0,
                                            long long t_fetch) {
+  ParamsRef p = uniform_params(pv);
   const int lane = lane_id();
   for (unsigned q = slot; q < nc; q += static_cast<unsigned>(p.n_workers)) {
     const long long t_item = p.trace ? wall_clock64() : 0;
@@ -869,8 +1023,21 @@ __device__ __noinline__ void combine_items(const Params& p, unsigned slot, unsig
 }
 
 // ---------------------------------------------------------------- worker loop
+// Nothing the tasks are called with lives in the wave's private memory: the
+// launch parameters are read in place (ParamsRef), a row tile travels as three
+// integers. A trip to private memory goes through the vector memory pipeline,
+// behind the weight loads of all eight waves, and cost every task several
+// microseconds (30B shape, T = 64: 263 -> 230 us without them).
+// disable_tail_calls: once no argument points into the caller's frame the
+// compiler marks the task calls as possible tail calls, and a function with such
+// a call site loses the treatment local functions get here (no callee-saved
+// registers, the caller knows what the callee clobbers): every task would save
+// and restore some fifty registers through private memory. The attribute
+// keeps the marks off.
 template <typename DT>
-__global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
+__global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_stream_kernel(
+    const Params params) {
+  ParamsRef p = kernel_params();
   __shared__ unsigned lds_flag[4];
   __shared__ unsigned lds_poller[4];
   if (threadIdx.x < 4) {
@@ -883,8 +1050,13 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
   const int waves_per_group = blockDim.x >> 6;
   Control* ctl = p.ctl;
   const unsigned T = static_cast<unsigned>(p.T);
-  const unsigned n_eg = static_cast<unsigned>((p.E + ROUTER_EXP - 1) / ROUTER_EXP);
-  const unsigned n_tg = (T + ROUTER_TOK - 1u) / ROUTER_TOK;
+  // dot tasks: 8 x 8 chains per wave, or (dot16) 16 x 16 per workgroup; those are
+  // not drawn, workgroup b < n_dot runs number b before its waves take tickets
+  const bool dot16 = p.dot16 != 0;
+  const unsigned dot_side = dot16 ? 16u : static_cast<unsigned>(ROUTER_EXP);
+  static_assert(ROUTER_EXP == ROUTER_TOK, "square dot tasks");
+  const unsigned n_eg = (static_cast<unsigned>(p.E) + dot_side - 1u) / dot_side;
+  const unsigned n_tg = (T + dot_side - 1u) / dot_side;
   const unsigned n_dot = n_tg * n_eg;
   const unsigned n_router = n_dot + T;  // dot tasks, then one select task per token
   const unsigned t_scan = n_router;
@@ -912,15 +1084,16 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
   // hands out the tickets after those.
   const unsigned n_workers = static_cast<unsigned>(p.n_workers);
   bool first = true;
-  unsigned first_tk = static_cast<unsigned>(wave_in_group) * gridDim.x + blockIdx.x;
-  unsigned dyn_base = n_workers;  // tickets below this are handed out statically
+  const unsigned n_skip = dot16 ? n_dot : 0u;
+  unsigned first_tk = n_skip + static_cast<unsigned>(wave_in_group) * gridDim.x + blockIdx.x;
+  unsigned dyn_base = n_skip + n_workers;  // tickets below this are handed out statically
   if (p.early) {
     // The other workers start streaming weights at once, and a routing task
     // whose loads queue behind those in its CU's memory pipeline runs a third
     // slower. So the routing tasks sit together on the first workgroups: dot
     // tasks on waves 0..3 (one per SIMD), select and scan tasks on waves 4..7.
     // Workers of those workgroups without a routing task take dynamic tickets.
-    const unsigned nr = max((n_dot + 3u) / 4u, (T + 4u) / 4u);
+    const unsigned nr = max(dot16 ? n_dot : (n_dot + 3u) / 4u, (T + 4u) / 4u);
     const unsigned rest = gridDim.x - nr;
     dyn_base = n_router + 1u + 8u * rest;
     if (blockIdx.x >= nr) {
@@ -929,11 +1102,26 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
       const unsigned q = blockIdx.x * 4u + (static_cast<unsigned>(wave_in_group) & 3u);
       if (wave_in_group < 4) {
         first_tk = q;
-        first = q < n_dot;
+        first = !dot16 && q < n_dot;
       } else {
         first_tk = n_dot + q;  // q == T: the scan
         first = q <= T;
       }
+    }
+  }
+
+  if (dot16 && blockIdx.x < n_dot) {
+    const long long t0 = p.trace ? wall_clock64() : 0;
+    router_dot16_task(p, static_cast<int>(blockIdx.x / n_eg), static_cast<int>(blockIdx.x % n_eg));
+    if (p.trace && threadIdx.x == 0 && blockIdx.x < p.trace_cap) {
+      const long long t1 = wall_clock64();
+      TraceRec* r = p.trace + blockIdx.x;
+      st16(r, u32x4{blockIdx.x, 0u, worker, blockIdx.x});
+      st16(reinterpret_cast<char*>(r) + 16,
+           u32x4{static_cast<unsigned>(t0), static_cast<unsigned>(t0 >> 32),
+                 static_cast<unsigned>(t0), static_cast<unsigned>(t0 >> 32)});
+      st16(reinterpret_cast<char*>(r) + 32,
+           u32x4{static_cast<unsigned>(t1), static_cast<unsigned>(t1 >> 32), 0u, 0u});
     }
   }
 
@@ -986,11 +1174,11 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
       tile.pad = 0;
       const int nblk = static_cast<int>(j % nt1);
       if (p.T <= 16) {
-        gateup_task<DT, 1, true>(p, tile, nblk);
+        gateup_task<DT, 1, true>(p, tile.expert, tile.row0, tile.rows, nblk);
       } else if (p.T <= 32) {
-        gateup_task<DT, 2, true>(p, tile, nblk);
+        gateup_task<DT, 2, true>(p, tile.expert, tile.row0, tile.rows, nblk);
       } else {
-        gateup_task<DT, 4, true>(p, tile, nblk);
+        gateup_task<DT, 4, true>(p, tile.expert, tile.row0, tile.rows, nblk);
       }
       wave_arrive(&p.g1_done[aux].v);
     } else {
@@ -1022,9 +1210,9 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
           }
           tile = ld_tile(&p.mtiles[aux]);
           if (tile.rows <= 32) {
-            gateup_task<DT, 2, false>(p, tile, nblk);
+            gateup_task<DT, 2, false>(p, tile.expert, tile.row0, tile.rows, nblk);
           } else {
-            gateup_task<DT, 4, false>(p, tile, nblk);
+            gateup_task<DT, 4, false>(p, tile.expert, tile.row0, tile.rows, nblk);
           }
         }
         wave_arrive(&p.g1_done[aux].v);
@@ -1039,11 +1227,11 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
         const TileDesc tile = ld_tile(&p.mtiles[aux]);
         const int nblk = static_cast<int>(j % nt1);
         if (tile.rows <= 16) {
-          gateup_task<DT, 1, false>(p, tile, nblk);
+          gateup_task<DT, 1, false>(p, tile.expert, tile.row0, tile.rows, nblk);
         } else if (tile.rows <= 32) {
-          gateup_task<DT, 2, false>(p, tile, nblk);
+          gateup_task<DT, 2, false>(p, tile.expert, tile.row0, tile.rows, nblk);
         } else {
-          gateup_task<DT, 4, false>(p, tile, nblk);
+          gateup_task<DT, 4, false>(p, tile.expert, tile.row0, tile.rows, nblk);
         }
         wave_arrive(&p.g1_done[aux].v);
       } else if (j < n1 + n2) {
@@ -1066,11 +1254,11 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
           }
           unsigned* dep = &p.g1_done[tile.expert].v;
           if (tile.rows <= 16) {
-            ok = down_task<DT, 1, true>(p, tile, nblk, dep, nt1);
+            ok = down_task<DT, 1, true>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           } else if (tile.rows <= 32) {
-            ok = down_task<DT, 2, true>(p, tile, nblk, dep, nt1);
+            ok = down_task<DT, 2, true>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           } else {
-            ok = down_task<DT, 4, true>(p, tile, nblk, dep, nt1);
+            ok = down_task<DT, 4, true>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           }
         } else {
           // the task reads its rows' gate weights and destinations up front
@@ -1082,11 +1270,11 @@ __global__ __launch_bounds__(512) void moe_stream_kernel(const Params p) {
           if (tile.rows == 0) {  // early mode keeps the tiles of unused experts
             ok = true;
           } else if (tile.rows <= 16) {
-            ok = down_task<DT, 1, false>(p, tile, nblk, dep, nt1);
+            ok = down_task<DT, 1, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           } else if (tile.rows <= 32) {
-            ok = down_task<DT, 2, false>(p, tile, nblk, dep, nt1);
+            ok = down_task<DT, 2, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           } else {
-            ok = down_task<DT, 4, false>(p, tile, nblk, dep, nt1);
+            ok = down_task<DT, 4, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           }
         }
         if (!ok) break;
