@@ -310,10 +310,10 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
 // The tiled variant needs bf16, tile-aligned shapes and token rows it can
 // address with 32-bit byte offsets. AUTO takes it once an expert sees about 24
 // rows on average when the packed weight copy exists (30B shape, us, streaming /
-// tiled: T=384 338 / 340, T=512 379 / 342; 235B shape: T=256 970 / 1018, T=512
-// 1119 / 1048), and from about 4 rows when the weights are read in the caller's
-// row-major layout, which the streaming variant reads poorly (30B: T=64 359 /
-// 352, T=128 411 / 358).
+// tiled: T=320 283 / 282, T=384 292 / 284, T=512 333 / 289; 235B shape: T=384
+// 920 / 945, T=512 1025 / 960), and from about 3 rows when the weights are read
+// in the caller's row-major layout, which the streaming variant reads poorly
+// (30B: T=32 272 / 270, T=48 296 / 283, T=64 312 / 291, T=128 363 / 297).
 static bool tiled_eligible(const FlashMoeLayerDesc& d, int tokens_num) {
   return d.dtype == FLASH_MOE_BF16 && d.hidden % 256 == 0 && d.intermediate % 128 == 0 &&
          tokens_num <= fmoe::tiled_max_tokens() &&
@@ -328,7 +328,7 @@ int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num) {
   if (d.sched == FLASH_MOE_SCHED_TILED) return FLASH_MOE_SCHED_TILED;
   const long long rows = static_cast<long long>(tokens_num) * d.top_k;
   const bool packed = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
-  return rows >= (packed ? 24ll : 4ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
+  return rows >= (packed ? 24ll : 3ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
 }
 
 int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int tokens_num,

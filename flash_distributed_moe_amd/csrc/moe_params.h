@@ -139,8 +139,7 @@ struct Params {
 // weight loads. A kernel that defines FMOE_PARAMS_IN_KERNARG before including
 // this header reads them in place in the kernel-argument segment instead
 // (constant address space): a field costs a scalar load that the scalar cache
-// serves. That is what short tasks want (the streaming variant); the tiled
-// variant's GEMM tasks have no register to spare for it and keep the copy.
+// serves. Both kernels do.
 #if defined(__HIP_DEVICE_COMPILE__) && defined(FMOE_PARAMS_IN_KERNARG)
 typedef const __attribute__((address_space(4))) Params& ParamsRef;
 #else

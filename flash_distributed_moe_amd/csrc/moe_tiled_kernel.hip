@@ -26,6 +26,7 @@
 // (src/hip/kernel/tasks/internal/gemmImpl/basicGemmTileImpl.h:14-94).
 #include <type_traits>
 
+#define FMOE_PARAMS_IN_KERNARG 1
 #include "moe_device.h"
 
 namespace fmoe {
@@ -79,7 +80,7 @@ struct WgShared {  // small static LDS block
 };
 
 // Thread 0 waits (bounded) for *p >= target; every thread learns the outcome.
-__device__ __forceinline__ bool wg_wait_ge(const Params& p, const unsigned* ptr, unsigned target,
+__device__ __forceinline__ bool wg_wait_ge(ParamsRef p, const unsigned* ptr, unsigned target,
                                            WgShared* sh) {
   if (threadIdx.x == 0) {
     unsigned ok = 1u;
@@ -108,7 +109,7 @@ __device__ __forceinline__ bool wg_wait_ge(const Params& p, const unsigned* ptr,
   return ok;
 }
 
-__device__ __forceinline__ bool wg_wait_flag(const Params& p, int which, WgShared* sh) {
+__device__ __forceinline__ bool wg_wait_flag(ParamsRef p, int which, WgShared* sh) {
   if (sh->flag[which] != 0u) return true;  // seen before by this workgroup
   const bool ok = wg_wait_ge(p, &p.wgflags[blockIdx.x].f[which], 1u, sh);
   if (ok && threadIdx.x == 0) sh->flag[which] = 1u;
@@ -136,7 +137,7 @@ __device__ __forceinline__ unsigned wg_arrive(unsigned* counter, WgShared* sh) {
   return old;
 }
 
-__device__ __forceinline__ void wg_broadcast_flag(const Params& p, int which) {
+__device__ __forceinline__ void wg_broadcast_flag(ParamsRef p, int which) {
   const int n = p.n_groups;
   WgFlags* flags = p.wgflags;
   for (int g = threadIdx.x; g < n; g += blockDim.x) st_relaxed(&flags[g].f[which], 1u);
@@ -194,7 +195,8 @@ constexpr int RT_EXP_BASE = RT_TOK_LOADS * 1024;     // byte offset of the exper
 constexpr int RT_STAGES = 4;
 static_assert(RT_EXP_BASE + 128 * RT_ROW_BYTES <= RT_STAGE_BYTES, "router stage too small");
 
-__device__ __noinline__ void tiled_router_task(const Params& p, int blk) {
+__device__ __noinline__ void tiled_router_task(ParamsRef pv, int blk) {
+  ParamsRef p = uniform_params(pv);
   const int T = uni(p.T), E = uni(p.E), H = uni(p.H);
   const unsigned char* tokens = uni(reinterpret_cast<const unsigned char*>(p.tokens));
   const unsigned char* gate = uni(reinterpret_cast<const unsigned char*>(p.gate));
@@ -362,7 +364,8 @@ __device__ __forceinline__ void load_to_lds_addr(const unsigned char* addr, unsi
                : "memory");
 }
 
-__device__ __noinline__ void tiled_router16_task(const Params& p, int blk) {
+__device__ __noinline__ void tiled_router16_task(ParamsRef pv, int blk) {
+  ParamsRef p = uniform_params(pv);
   const int T = uni(p.T), E = uni(p.E), H = uni(p.H);
   const unsigned char* tokens = uni(reinterpret_cast<const unsigned char*>(p.tokens));
   const unsigned char* gate = uni(reinterpret_cast<const unsigned char*>(p.gate));
@@ -484,7 +487,8 @@ __device__ __noinline__ void tiled_router16_task(const Params& p, int blk) {
 // Final scan: one wave turns the totals into row offsets and the row-tile table.
 constexpr int SCAN_EXPERTS = T_THREADS / 64;  // experts per expert-scan task
 
-__device__ __noinline__ void tiled_expert_scan_task(const Params& p, int blk) {
+__device__ __noinline__ void tiled_expert_scan_task(ParamsRef pv, int blk) {
+  ParamsRef p = uniform_params(pv);
   const int E = uni(p.E), W = uni(p.W), T = uni(p.T);
   const unsigned long long* masks = uni(p.masks);
   int* word_prefix = uni(p.word_prefix);
@@ -504,7 +508,8 @@ __device__ __noinline__ void tiled_expert_scan_task(const Params& p, int blk) {
   if (lane == 0) stc(&expert_count[e], base);
 }
 
-__device__ __noinline__ void tiled_scan_task(const Params& p) {
+__device__ __noinline__ void tiled_scan_task(ParamsRef pv) {
+  ParamsRef p = uniform_params(pv);
   const RouteTables r = route_tables(p);
   const int tid = threadIdx.x;
   if (tid < 64) {
@@ -554,7 +559,7 @@ __device__ __noinline__ void tiled_scan_task(const Params& p) {
   wg_broadcast_flag(p, FLAG_SCAN);
 }
 
-__device__ void tiled_scatter_task(const Params& p, int blk) {
+__device__ void tiled_scatter_task(ParamsRef p, int blk) {
   const RouteTables r = route_tables(p);
   const int i0 = blk * RT_TOK * r.K;
   const int n = min(RT_TOK * r.K, r.T * r.K - i0);
@@ -783,7 +788,8 @@ __device__ __forceinline__ size_t tiled_h_tile_bytes(int I) { return static_cast
 
 // gate/up: h[row, n0 .. n0+128) for one row tile
 // (test/singleGPU/cpp/moe/reference/refExpertFFN1.h:51-65).
-__device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& tile_in, int m, int nblk) {
+__device__ __noinline__ void tiled_gateup_task(ParamsRef pv, const TileDesc& tile_in, int m, int nblk) {
+  ParamsRef p = uniform_params(pv);
   const int H = uni(p.H), I = uni(p.I), K = uni(p.K);
   TileDesc tile;
   tile.expert = uni(tile_in.expert);
@@ -878,7 +884,8 @@ __device__ __noinline__ void tiled_gateup_task(const Params& p, const TileDesc& 
 
 // down: y[t*K+slot, n0 .. n0+256) = w * (h[row] . W2[e]^T)
 // (refFullMoe.h:58-65, src/hip/kernel/tasks/ffn2Task.h:37-40).
-__device__ __noinline__ void tiled_down_task(const Params& p, const TileDesc& tile_in, int m, int nblk) {
+__device__ __noinline__ void tiled_down_task(ParamsRef pv, const TileDesc& tile_in, int m, int nblk) {
+  ParamsRef p = uniform_params(pv);
   const int H = uni(p.H), I = uni(p.I);
   TileDesc tile;
   tile.expert = uni(tile_in.expert);
@@ -1127,7 +1134,8 @@ __device__ __forceinline__ int tall_token_block(int q) {
   return L < TALL_TM / 16 ? L : -1;
 }
 
-__device__ __noinline__ void tall_gateup_task(const Params& p, const TileDesc& tile_in, int m, int nblk) {
+__device__ __noinline__ void tall_gateup_task(ParamsRef pv, const TileDesc& tile_in, int m, int nblk) {
+  ParamsRef p = uniform_params(pv);
   const int H = uni(p.H), I = uni(p.I), K = uni(p.K);
   TileDesc tile;
   tile.expert = uni(tile_in.expert);
@@ -1213,7 +1221,8 @@ __device__ __noinline__ void tall_gateup_task(const Params& p, const TileDesc& t
   }
 }
 
-__device__ __noinline__ void tall_down_task(const Params& p, const TileDesc& tile_in, int m, int nblk) {
+__device__ __noinline__ void tall_down_task(ParamsRef pv, const TileDesc& tile_in, int m, int nblk) {
+  ParamsRef p = uniform_params(pv);
   const int H = uni(p.H), I = uni(p.I);
   TileDesc tile;
   tile.expert = uni(tile_in.expert);
@@ -1311,7 +1320,8 @@ __device__ __noinline__ void tall_down_task(const Params& p, const TileDesc& til
 
 // combine: out[t] = sum over slots, in slot order, of y[t*K+slot]
 // (refFullMoe.h:35,62-65).
-__device__ __noinline__ void tiled_combine_task(const Params& p, int blk) {
+__device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
+  ParamsRef p = uniform_params(pv);
   const int H = uni(p.H), K = uni(p.K), T = uni(p.T), E = uni(p.E), W = uni(p.W);
   unsigned short* out = uni(reinterpret_cast<unsigned short*>(p.out));
   const unsigned short* y = uni(reinterpret_cast<const unsigned short*>(p.y));
@@ -1378,7 +1388,11 @@ __device__ __forceinline__ int xcc_id() {
   return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 7;
 }
 
-__global__ __launch_bounds__(T_THREADS) void moe_tiled_kernel(const Params p) {
+// The launch parameters are read in place and the task calls keep the local
+// calling convention, as in the streaming variant (see its worker loop).
+__global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void moe_tiled_kernel(
+    const Params params) {
+  ParamsRef p = kernel_params();
   __shared__ WgShared sh;
   if (threadIdx.x == 0) {
     sh.ticket = 0u;
