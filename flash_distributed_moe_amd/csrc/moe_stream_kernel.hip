@@ -844,12 +844,16 @@ __device__ __noinline__ void gateup_task(ParamsRef pv, int expert, int row0, int
   gateup_body<DT, RB, DENSE, false>(p, tile, nblk, nullptr, nullptr);
 }
 
-// tile.expert is set on entry; the rest of the descriptor is filled in once the
-// routing is known
+// the rows of the expert's tile are worked out inside, once the routing is known
 template <typename DT>
-__device__ __noinline__ int gateup_early_task(ParamsRef pv, TileDesc& tile, int nblk,
+__device__ __noinline__ int gateup_early_task(ParamsRef pv, int expert, int nblk,
                                               unsigned* lds_flag, unsigned* lds_poller) {
   ParamsRef p = uniform_params(pv);
+  TileDesc tile;
+  tile.expert = expert;
+  tile.row0 = 0;
+  tile.rows = 0;
+  tile.pad = 0;
   return gateup_body<DT, 1, false, true>(p, tile, nblk, lds_flag, lds_poller);
 }
 
@@ -1087,6 +1091,7 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
   const unsigned n_skip = dot16 ? n_dot : 0u;
   unsigned first_tk = n_skip + static_cast<unsigned>(wave_in_group) * gridDim.x + blockIdx.x;
   unsigned dyn_base = n_skip + n_workers;  // tickets below this are handed out statically
+  unsigned late_lo = 0xFFFFFFFFu, late_skip = 0u;  // early mode: static tickets [late_lo, late_lo + late_skip)
   if (p.early) {
     // The other workers start streaming weights at once, and a routing task
     // whose loads queue behind those in its CU's memory pipeline runs a third
@@ -1096,8 +1101,20 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
     const unsigned nr = max(dot16 ? n_dot : (n_dot + 3u) / 4u, (T + 4u) / 4u);
     const unsigned rest = gridDim.x - nr;
     dyn_base = n_router + 1u + 8u * rest;
+    if (n1 >= 8u * rest) {
+      late_skip = 4u * rest;
+      late_lo = t_dyn0 + n1 - late_skip;
+      dyn_base = t_dyn0 + late_skip;
+    }
     if (blockIdx.x >= nr) {
       first_tk = n_router + 1u + static_cast<unsigned>(wave_in_group) * rest + (blockIdx.x - nr);
+      // A CU's waves 4..7 stream at half the rate of waves 0..3 while both run, so
+      // their first tasks end last of all (140-155 us against 70-80 at T = 64 on
+      // the 30B shape). They take the gate/up tasks of the last experts, whose down
+      // tasks are drawn last anyway; the tickets in between are drawn by the waves
+      // that finish first.
+      if (late_skip != 0u && wave_in_group >= 4)
+        first_tk = late_lo + (static_cast<unsigned>(wave_in_group) - 4u) * rest + (blockIdx.x - nr);
     } else {
       const unsigned q = blockIdx.x * 4u + (static_cast<unsigned>(wave_in_group) & 3u);
       if (wave_in_group < 4) {
@@ -1131,6 +1148,7 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
     if (!first) {
       if (lane == 0) tk = dyn_base + add_relaxed(&ctl->ticket.v, 1u);
       tk = __builtin_amdgcn_readfirstlane(tk);
+      if (tk >= late_lo) tk += late_skip;  // early mode: over the late waves' static tickets
     }
     first = false;
     unsigned kind = 0, aux = 0;
@@ -1201,7 +1219,7 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
         tile.row0 = 0;
         tile.rows = 0;
         tile.pad = 0;
-        const int st = gateup_early_task<DT>(p, tile, nblk, lds_flag, lds_poller);
+        const int st = gateup_early_task<DT>(p, tile.expert, nblk, lds_flag, lds_poller);
         if (st == 1) break;
         if (st == 2) {
           if (!perm_ready) {
@@ -1317,7 +1335,9 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
   }
   last = __builtin_amdgcn_readfirstlane(last);
   if (last) {
-    unsigned nm = min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
+    // (early mode: one row tile per expert, known without a trip to memory)
+    unsigned nm = p.early ? static_cast<unsigned>(p.E)
+                          : min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
     if (dense) nm = max(nm, static_cast<unsigned>(p.E));  // counters are per expert there
     for (unsigned i = lane; i < nm; i += 64) stc(&p.g1_done[i].v, 0u);
     for (int g = lane; g < p.n_groups; g += 64) {
