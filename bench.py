@@ -39,8 +39,8 @@ BOUND = {
 # packed weight copy; other workloads have no measurement. For the decode kernel the read counter
 # is a lower bound (it under-counts wide streaming reads: it stays below the weight bytes).
 MEASURED_TRAFFIC = {
-    "qwen3_30b_decode": (588379 + 8513) * 1024,
-    "qwen3_30b_prefill": (1102202 + 429478) * 1024,
+    "qwen3_30b_decode": (587847 + 6016) * 1024,
+    "qwen3_30b_prefill": (1113843 + 429478) * 1024,
 }
 
 

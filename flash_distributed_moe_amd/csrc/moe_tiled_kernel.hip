@@ -75,6 +75,7 @@ __device__ __forceinline__ T* uni(T* ptr) {
 
 struct WgShared {  // small static LDS block
   unsigned ticket;
+  unsigned next;
   unsigned ok;
   unsigned flag[4];
 };
@@ -133,6 +134,25 @@ __device__ __forceinline__ unsigned wg_arrive(unsigned* counter, WgShared* sh) {
   }
   __syncthreads();
   const unsigned old = sh->ticket;
+  __syncthreads();
+  return old;
+}
+
+// The same, and the workgroup's next ticket from `queue` in the same trip to
+// memory: thread 0 sends both atomics before it looks at either result.
+__device__ __forceinline__ unsigned wg_arrive_and_draw(unsigned* counter, unsigned* queue,
+                                                       unsigned& next, WgShared* sh) {
+  fence_release();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned old = add_relaxed(counter, 1u);
+    const unsigned nxt = add_relaxed(queue, 1u);
+    sh->ticket = old;
+    sh->next = nxt;
+  }
+  __syncthreads();
+  const unsigned old = sh->ticket;
+  next = sh->next;
   __syncthreads();
   return old;
 }
@@ -1490,12 +1510,14 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
     const unsigned lo = nm * q / 8u, hi = nm * (q + 1u) / 8u;
     const unsigned tiles = hi - lo;
     const unsigned q1 = tiles * nt1, q2 = tiles * nt2;
+    // the first ticket of a queue is drawn on its own, the others together with the
+    // arrival of the task before
+    if (threadIdx.x == 0) sh.ticket = add_relaxed(&ctl->xq[q].v, 1u);
+    __syncthreads();
+    unsigned j = sh.ticket;
+    __syncthreads();
     while (ok) {
       const long long t_fetch = p.trace ? wall_clock64() : 0;
-      if (threadIdx.x == 0) sh.ticket = add_relaxed(&ctl->xq[q].v, 1u);
-      __syncthreads();
-      const unsigned j = sh.ticket;
-      __syncthreads();
       if (j >= q1 + q2) break;
       long long t_ready = 0;
       if (j < q1) {
@@ -1507,21 +1529,23 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
         } else {
           tiled_gateup_task(p, tile, static_cast<int>(m), static_cast<int>(j % nt1));
         }
-        wg_arrive<false>(&p.g1_done[m].v, &sh);
-        trace(t_dyn0 + lo * nt1 + j, 3, m, t_fetch, t_ready);
+        const unsigned done = j;
+        wg_arrive_and_draw(&p.g1_done[m].v, &ctl->xq[q].v, j, &sh);
+        trace(t_dyn0 + lo * nt1 + done, 3, m, t_fetch, t_ready);
       } else {
         const unsigned jj = j - q1;
         const unsigned m = lo + jj / nt2;
+        const TileDesc tile = ld_tile(&p.mtiles[m]);  // in flight while thread 0 looks at the counter
         ok = wg_wait_ge(p, &p.g1_done[m].v, nt1, &sh);
         if (ok) {
           if (p.trace) t_ready = wall_clock64();
-          const TileDesc tile = ld_tile(&p.mtiles[m]);
           if (tile.rows > TM) {
             tall_down_task(p, tile, static_cast<int>(m), static_cast<int>(jj % nt2));
           } else {
             tiled_down_task(p, tile, static_cast<int>(m), static_cast<int>(jj % nt2));
           }
-          if (wg_arrive<false>(&ctl->g2_done.v, &sh) == n2_total - 1u) wg_broadcast_flag(p, FLAG_G2);
+          if (wg_arrive_and_draw(&ctl->g2_done.v, &ctl->xq[q].v, j, &sh) == n2_total - 1u)
+            wg_broadcast_flag(p, FLAG_G2);
           trace(t_dyn0 + nm * nt1 + lo * nt2 + jj, 4, m, t_fetch, t_ready);
         }
       }
