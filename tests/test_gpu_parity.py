@@ -85,6 +85,23 @@ def test_odd_shapes(shape):
     run_case(synth.MoeConfig("odd", T, H, E, k, I, dt), seed=T + H)
 
 
+@pytest.mark.parametrize("shape", [
+    # T, H, E, k, I, hot: bf16 layers with H % 256 == 0 run the logit chains on the
+    # matrix core, 16 tokens x 16 experts per workgroup, in stages of 256 k whose
+    # loads go out eight stages at a time
+    (17, 768, 24, 3, 64, 0),      # three stages; last token group and last expert group partly empty
+    (65, 2304, 60, 5, 96, 0),     # nine stages: a second, short batch of loads
+    (130, 512, 200, 6, 160, 0),   # 9 x 13 groups
+    (1, 4096, 16, 2, 64, 0),      # one token, sixteen stages
+    (200, 1024, 48, 4, 64, 3),    # router bias
+    (40, 768, 24, 3, 64, 0),      # early gate/up tasks (T <= 64, T*k >= E) behind the same router
+    (64, 512, 72, 8, 32, 2),      # the same with 4.5 expert groups and a bias
+])
+def test_matrix_core_router_shapes(shape):
+    T, H, E, k, I, hot = shape
+    run_case(synth.MoeConfig("mcr", T, H, E, k, I, "bf16", hot=hot), seed=T + E)
+
+
 def test_router_bias_hot_experts_small():
     cfg = synth.MoeConfig("hot", 256, 256, 16, 4, 64, "bf16", hot=2)
     run_case(cfg, seed=3)
