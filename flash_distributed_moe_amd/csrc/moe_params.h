@@ -32,7 +32,7 @@ constexpr int ROUTER_TOK = 8;    // streaming variant: tokens per router dot tas
 constexpr int ROUTER_EXP = 8;    // streaming variant: experts per router dot task
 constexpr int DOT16_KC = 256;    // streaming variant, matrix-core router: k per LDS stage
 constexpr int SCAN_LDS_WORDS = 1024;  // mask words (experts x 64-token words) the small-batch scan keeps in LDS
-constexpr int EARLY_MAX_TOKENS = 64;   // batches up to this size take their gate/up weights before the routing is known
+constexpr int EARLY_MAX_TOKENS = 192;  // batches up to this size may take their gate/up weights before the routing is known
 constexpr int MAX_EXPERTS = 256;  // experts are spread 64 per wave register slot
 constexpr int MAX_TOPK = 32;
 

@@ -695,7 +695,7 @@ struct RoundSteps {
 // entries i = token*K + slot that name e, in ascending i (the order the
 // permutation gives them), and its first row is the number of entries that name
 // a lower expert. Lanes 0..15 (and their copies in the other lane groups) get
-// the entry of row min(lane & 15, rows - 1). For batches of at most 64 tokens.
+// the entry of row min(lane & 15, rows - 1). The table is read 512 entries at a time.
 __device__ __forceinline__ void tile_from_topk(ParamsRef p, int e, int& row0, int& rows,
                                                int& entry) {
   const int lane = lane_id();

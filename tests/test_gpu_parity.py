@@ -96,6 +96,8 @@ def test_odd_shapes(shape):
     (200, 1024, 48, 4, 64, 3),    # router bias
     (40, 768, 24, 3, 64, 0),      # early gate/up tasks (T <= 64, T*k >= E) behind the same router
     (64, 512, 72, 8, 32, 2),      # the same with 4.5 expert groups and a bias
+    (60, 256, 16, 2, 64, 2),      # early tasks; the two hot experts hold far more than 16 rows and start over
+    (150, 512, 128, 8, 64, 0),    # early tasks behind three 64-token mask words
 ])
 def test_matrix_core_router_shapes(shape):
     T, H, E, k, I, hot = shape
