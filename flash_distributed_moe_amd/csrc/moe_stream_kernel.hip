@@ -486,7 +486,8 @@ __device__ __noinline__ void scan_scatter_small_task(ParamsRef pv) {
     }
     const int incl = wave_inclusive_scan(c);
     const int off = base + incl - c;
-    // early mode: expert e owns tile e, empty or not (c <= 64 there)
+    // early mode: expert e owns tile e, empty or not, and the tile holds all of the
+    // expert's rows (the tasks walk through it SKINNY_MT rows at a time)
     const int nt = p.early ? (e < r.E ? 1 : 0) : (c + SKINNY_MT - 1) / SKINNY_MT;
     const int tincl = wave_inclusive_scan(nt);
     const int toff = tile_base + tincl - nt;
@@ -498,7 +499,7 @@ __device__ __noinline__ void scan_scatter_small_task(ParamsRef pv) {
         if (toff + i < r.max_mtiles) {
           stc16(&r.mtiles[toff + i],
                 make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + i * SKINNY_MT),
-                           static_cast<unsigned>(min(SKINNY_MT, c - i * SKINNY_MT)), 0u));
+                           static_cast<unsigned>(p.early ? c : min(SKINNY_MT, c - i * SKINNY_MT)), 0u));
         }
       }
     }
@@ -1227,10 +1228,15 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
             perm_ready = true;
           }
           tile = ld_tile(&p.mtiles[aux]);
-          if (tile.rows <= 32) {
-            gateup_task<DT, 2, false>(p, tile.expert, tile.row0, tile.rows, nblk);
-          } else {
-            gateup_task<DT, 4, false>(p, tile.expert, tile.row0, tile.rows, nblk);
+          for (int r0 = 0; r0 < tile.rows; r0 += SKINNY_MT) {
+            const int rc = min(SKINNY_MT, tile.rows - r0);
+            if (rc <= 16) {
+              gateup_task<DT, 1, false>(p, tile.expert, tile.row0 + r0, rc, nblk);
+            } else if (rc <= 32) {
+              gateup_task<DT, 2, false>(p, tile.expert, tile.row0 + r0, rc, nblk);
+            } else {
+              gateup_task<DT, 4, false>(p, tile.expert, tile.row0 + r0, rc, nblk);
+            }
           }
         }
         wave_arrive(&p.g1_done[aux].v);
@@ -1285,14 +1291,28 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
             perm_ready = true;
           }
           unsigned* dep = &p.g1_done[aux].v;
-          if (tile.rows == 0) {  // early mode keeps the tiles of unused experts
+          // early mode keeps the tiles of unused experts (no rows) and gives an expert
+          // one tile however many rows it holds; otherwise this is a single pass
+          if (tile.rows == 0) {
             ok = true;
           } else if (tile.rows <= 16) {
             ok = down_task<DT, 1, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           } else if (tile.rows <= 32) {
             ok = down_task<DT, 2, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
-          } else {
+          } else if (tile.rows <= SKINNY_MT) {
             ok = down_task<DT, 4, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
+          } else {
+            ok = true;
+            for (int r0 = 0; ok && r0 < tile.rows; r0 += SKINNY_MT) {
+              const int rc = min(SKINNY_MT, tile.rows - r0);
+              if (rc <= 16) {
+                ok = down_task<DT, 1, false>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+              } else if (rc <= 32) {
+                ok = down_task<DT, 2, false>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+              } else {
+                ok = down_task<DT, 4, false>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+              }
+            }
           }
         }
         if (!ok) break;

@@ -98,6 +98,8 @@ def test_odd_shapes(shape):
     (64, 512, 72, 8, 32, 2),      # the same with 4.5 expert groups and a bias
     (60, 256, 16, 2, 64, 2),      # early tasks; the two hot experts hold far more than 16 rows and start over
     (150, 512, 128, 8, 64, 0),    # early tasks behind three 64-token mask words
+    (150, 256, 64, 4, 64, 1),     # early tasks; the hot expert holds all 150 tokens: its one tile is walked in 64-row steps
+    (100, 512, 128, 8, 32, 2),    # the same with two hot experts of 100 rows
 ])
 def test_matrix_core_router_shapes(shape):
     T, H, E, k, I, hot = shape
