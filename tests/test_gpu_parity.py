@@ -130,6 +130,28 @@ def test_relaunch_and_smaller_batch():
         case.close()
 
 
+@pytest.mark.parametrize("sched", [_lib.SCHED_STREAM, _lib.SCHED_AUTO])
+def test_relaunch_across_batch_sizes(sched):
+    """One launcher, batches that take different paths one after the other (early
+    gate/up tasks, the ordinary ticket order, one token, and with AUTO the tiled
+    variant): every launch leaves the counters as the next one needs them."""
+    cfg = synth.MoeConfig("seq", 600, 512, 64, 4, 128, "bf16")
+    case = GpuCase(cfg, seed=11, sched=sched)
+    try:
+        x = case.inp["tokens"]
+        full = case.run()
+        case.check_routing(x, case.launcher.routing(cfg.T))
+        case.check_outputs(x, full, np.arange(0, cfg.T, 7))
+        for T in (150, 600, 40, 1, 190, 300, 64):
+            part = x[:T].contiguous()
+            out = case.run(tokens=part)
+            case.check_routing(part, case.launcher.routing(T))
+            case.check_outputs(part, out, np.arange(0, T, 3))
+        assert case.launcher.status()[0] == 0
+    finally:
+        case.close()
+
+
 @pytest.mark.parametrize("shape", [
     # T, H, E, k, I: the tiled (MFMA 32x32, LDS-staged) variant forced on small problems
     (300, 256, 8, 2, 128),      # ragged last row tile (75 rows per expert on average)
