@@ -198,17 +198,17 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   // T=8 167 / 145 us, T=16 199 / 200, T=24 227 / 242, T=64 263 / 278).
   const bool reaches_experts =
       static_cast<long long>(T) * d.top_k >= static_cast<long long>(d.experts);
-  // An early task serves one block of 16 rows; a tile with more starts over from
-  // the tile table once the scan is done. So: at most 12 rows per expert on
-  // average (30B shape, with / without: T=80 230 / 243 us, T=128 242 / 253,
-  // T=192 263 / 266).
-  const bool few_rows =
-      static_cast<long long>(T) * d.top_k <= 12ll * static_cast<long long>(d.experts);
-  p.early = (reaches_experts && few_rows && !p.dense && p.fuse_scatter &&
+  // An early task serves one block of 16 rows, or two; a tile with more starts
+  // over from the tile table once the scan is done. So: one block up to 12 rows
+  // per expert on average (30B shape, with / without: T=80 230 / 243 us, T=128
+  // 242 / 253, T=192 263 / 266), two up to 24.
+  const long long slots = static_cast<long long>(T) * d.top_k;
+  const int early_blocks = slots <= 12ll * d.experts ? 1 : slots <= 24ll * d.experts ? 2 : 0;
+  p.early = (reaches_experts && early_blocks != 0 && !p.dense && p.fuse_scatter &&
              T <= fmoe::EARLY_MAX_TOKENS &&
              d.experts * ((T + 63) / 64) <= fmoe::SCAN_LDS_WORDS && d.experts <= L.max_mtiles &&
              routing_groups <= p.n_groups / 2)
-                ? 1
+                ? early_blocks
                 : 0;
   p.tpad = (T + 15) / 16 * 16;
   p.max_mtiles = L.max_mtiles;

@@ -32,7 +32,7 @@ constexpr int ROUTER_TOK = 8;    // streaming variant: tokens per router dot tas
 constexpr int ROUTER_EXP = 8;    // streaming variant: experts per router dot task
 constexpr int DOT16_KC = 256;    // streaming variant, matrix-core router: k per LDS stage
 constexpr int SCAN_LDS_WORDS = 1024;  // mask words (experts x 64-token words) the small-batch scan keeps in LDS
-constexpr int EARLY_MAX_TOKENS = 192;  // batches up to this size may take their gate/up weights before the routing is known
+constexpr int EARLY_MAX_TOKENS = 384;  // batches up to this size may take their gate/up weights before the routing is known
 constexpr int MAX_EXPERTS = 256;  // experts are spread 64 per wave register slot
 constexpr int MAX_TOPK = 32;
 
@@ -124,7 +124,7 @@ struct Params {
   int n_groups;                    // workgroups in the grid
   int fuse_scatter;                // 1: the scan task also writes the permutation
   int dense;                       // 1: gate/up runs for every (expert, token) pair (small batches)
-  int early;                       // 1: row tile e belongs to expert e (empty or not), so gate/up tasks are
+  int early;                       // 1, 2: row tile e belongs to expert e (empty or not), so gate/up tasks are
                                    //    handed out at launch and fetch their first weights under the routing
   int tpad;                        // dense mode: h rows reserved per expert
   int dot16;                       // 1 (streaming variant, bf16): the logit chains run on the matrix core, 16 tokens x

@@ -697,12 +697,16 @@ struct RoundSteps {
 // permutation gives them), and its first row is the number of entries that name
 // a lower expert. Lanes 0..15 (and their copies in the other lane groups) get
 // the entry of row min(lane & 15, rows - 1). The table is read 512 entries at a time.
+template <int RB>
 __device__ __forceinline__ void tile_from_topk(ParamsRef p, int e, int& row0, int& rows,
-                                               int& entry) {
+                                               int (&entry)[RB]) {
   const int lane = lane_id();
   const int r16 = lane & 15;
   const int n = p.T * p.K;
-  int cnt = 0, lt = 0, idx = 0;
+  int cnt = 0, lt = 0;
+  int idx[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) idx[r] = 0;
   constexpr int B = 8;  // entries per lane in flight together
   for (int i0 = 0; i0 < n; i0 += 64 * B) {
     int ee[B];
@@ -716,17 +720,32 @@ __device__ __forceinline__ void tile_from_topk(ParamsRef p, int e, int& row0, in
       const unsigned long long m = __ballot(ee[b] == e);
       lt += __popcll(__ballot(ee[b] >= 0 && ee[b] < e));
       const int pc = __popcll(m);
-      if (r16 >= cnt && r16 < cnt + pc) {
-        unsigned long long mm = m;
-        for (int j = cnt; j < r16; ++j) mm &= mm - 1ull;
-        idx = i0 + 64 * b + static_cast<int>(__builtin_ctzll(mm));
+#pragma unroll
+      for (int r = 0; r < RB; ++r) {
+        const int want = r * 16 + r16;  // this lane keeps the entries of rows r16, 16 + r16, ...
+        if (want >= cnt && want < cnt + pc) {
+          unsigned long long mm = m;
+          for (int j = cnt; j < want; ++j) mm &= mm - 1ull;
+          idx[r] = i0 + 64 * b + static_cast<int>(__builtin_ctzll(mm));
+        }
       }
       cnt += pc;
     }
   }
   row0 = lt;
   rows = cnt;
-  entry = __shfl(idx, max(min(r16, cnt - 1), 0), 64);
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    // row r*16 + r16, or the last row when the tile is shorter: held by lane (row % 16) as entry row / 16
+    const int row = max(min(r * 16 + r16, cnt - 1), 0);
+    int v = 0;
+#pragma unroll
+    for (int q = 0; q < RB; ++q) {
+      const int got = __shfl(idx[q], row & 15, 64);
+      if ((row >> 4) == q) v = got;
+    }
+    entry[r] = v;
+  }
 }
 
 // EARLY (small batches: every expert owns the row tile of its own index, empty
@@ -787,19 +806,20 @@ __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk
   int status = 0;
   const bool ran = stream_mma<DT, NA, RB, U, false>(ap, bp, p.H / (4 * EPV), astep, acc, [&] {
     if (EARLY) {
-      static_assert(!EARLY || RB == 1, "tile_from_topk serves one block of 16 rows");
       if (!wait_flag(p, FLAG_ROUTED, lds_flag, lds_poller)) {
         status = 1;
         return false;
       }
-      int entry;
-      tile_from_topk(p, tile.expert, tile.row0, tile.rows, entry);
+      int entry[RB];
+      tile_from_topk<RB>(p, tile.expert, tile.row0, tile.rows, entry);
       if (tile.rows == 0) return false;
       if (tile.rows > 16 * RB) {
         status = 2;
         return false;
       }
-      bp[0] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(entry / p.K) * p.H + g * EPV;
+#pragma unroll
+      for (int r = 0; r < RB; ++r)
+        bp[r] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(entry[r] / p.K) * p.H + g * EPV;
     }
     return true;
   });
@@ -846,7 +866,7 @@ __device__ __noinline__ void gateup_task(ParamsRef pv, int expert, int row0, int
 }
 
 // the rows of the expert's tile are worked out inside, once the routing is known
-template <typename DT>
+template <typename DT, int RB>
 __device__ __noinline__ int gateup_early_task(ParamsRef pv, int expert, int nblk,
                                               unsigned* lds_flag, unsigned* lds_poller) {
   ParamsRef p = uniform_params(pv);
@@ -855,7 +875,7 @@ __device__ __noinline__ int gateup_early_task(ParamsRef pv, int expert, int nblk
   tile.row0 = 0;
   tile.rows = 0;
   tile.pad = 0;
-  return gateup_body<DT, 1, false, true>(p, tile, nblk, lds_flag, lds_poller);
+  return gateup_body<DT, RB, false, true>(p, tile, nblk, lds_flag, lds_poller);
 }
 
 // ----------------------------------------------------------------------- down
@@ -1220,7 +1240,10 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
         tile.row0 = 0;
         tile.rows = 0;
         tile.pad = 0;
-        const int st = gateup_early_task<DT>(p, tile.expert, nblk, lds_flag, lds_poller);
+        // (p.early is the number of 16-row blocks an early task carries)
+        const int st = p.early == 1
+                           ? gateup_early_task<DT, 1>(p, tile.expert, nblk, lds_flag, lds_poller)
+                           : gateup_early_task<DT, 2>(p, tile.expert, nblk, lds_flag, lds_poller);
         if (st == 1) break;
         if (st == 2) {
           if (!perm_ready) {

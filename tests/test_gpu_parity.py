@@ -100,6 +100,8 @@ def test_odd_shapes(shape):
     (150, 512, 128, 8, 64, 0),    # early tasks behind three 64-token mask words
     (150, 256, 64, 4, 64, 1),     # early tasks; the hot expert holds all 150 tokens: its one tile is walked in 64-row steps
     (100, 512, 128, 8, 32, 2),    # the same with two hot experts of 100 rows
+    (250, 512, 128, 8, 64, 0),    # 12 to 24 rows per expert: early tasks of two row blocks
+    (230, 256, 64, 4, 64, 1),     # the same with a hot expert of 230 rows
 ])
 def test_matrix_core_router_shapes(shape):
     T, H, E, k, I, hot = shape
