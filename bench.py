@@ -35,12 +35,14 @@ BOUND = {
 
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
-# dispatch, copy-kernel factor 1.000) on exactly these workloads with the default seed and the
-# packed weight copy; other workloads have no measurement. For the decode kernel the read counter
-# is a lower bound (it under-counts wide streaming reads: it stays below the weight bytes).
+# dispatch) on exactly these workloads with the default seed and the packed weight copy; other
+# workloads have no measurement. Each counter is scaled by what it reads for a plain copy of
+# 1 GiB: WRITE_SIZE 1.000, FETCH_SIZE 0.500 (this chip reads HBM in 128-byte requests, which
+# the counter's formula prices at 64 bytes each).
+FETCH_SCALE = 0.5
 MEASURED_TRAFFIC = {
-    "qwen3_30b_decode": (587847 + 6016) * 1024,
-    "qwen3_30b_prefill": (1113843 + 429478) * 1024,
+    "qwen3_30b_decode": int(587847 / FETCH_SCALE + 6016) * 1024,
+    "qwen3_30b_prefill": int(1113843 / FETCH_SCALE + 429478) * 1024,
 }
 
 
@@ -107,6 +109,9 @@ def main():
     ap.add_argument("--sched", type=int, default=0)
     ap.add_argument("--no-pack-weights", action="store_true",
                     help="read the caller's weight layout instead of the packed second copy")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only copy 1 GiB device to device five times: the known traffic the "
+                         "rocprofv3 byte counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs the MoE layer on ONE GPU (no collectives, no "
@@ -119,6 +124,15 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    if args.copy_calibration:
+        a = torch.randn(1 << 28, device="cuda:0", dtype=torch.float32)
+        b = torch.empty_like(a)
+        for _ in range(5):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"copies": 5, "kib_read_each": 1 << 20,
+                                               "kib_written_each": 1 << 20}}))
+        return
     cfg = synth.CONFIGS[args.config]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
