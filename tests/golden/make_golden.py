@@ -43,7 +43,7 @@ def main():
     if not oracle.have_ref():
         oracle.build(ref=True)
 
-    # 1. BASELINE config 1 (tiny fp32), whole layer.
+    # 1. the reference's own CPU-runnable case (tiny fp32), whole layer.
     cfg = synth.CONFIGS["tiny_f32"]
     inp = synth.make_inputs_np(cfg, seed=7907)
     out = oracle.ref_full_moe(inp["tokens"], inp["gate"], inp["ffn1"], inp["ffn2"], cfg.k)
