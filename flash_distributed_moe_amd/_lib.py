@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libflashMoe.so")
 F32, BF16 = 0, 1
 SCHED_AUTO, SCHED_STREAM, SCHED_TILED = 0, 1, 2
 FLAG_PACK_WEIGHTS = 1
+NOALLOC_SCRATCH_BYTES = 64 << 20
 HIP_SUCCESS = 0
 HIP_ERROR_INVALID_VALUE = 1
 HIP_ERROR_UNKNOWN = 999
@@ -45,6 +46,8 @@ C_ABI = {
     "flashMoeRefreshWeights": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p]),
     "flashMoeLaunch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                       ctypes.c_int, ctypes.c_void_p]),
+    "flashMoeLaunchNoAlloc": (ctypes.c_int, [ctypes.POINTER(LayerDesc), ctypes.c_void_p,
+                                             ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]),
     "flashMoeDestroy": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p]),
     "flashMoeReadRouting": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
                                            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,

@@ -15,6 +15,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "../../include/iMoeKernelLauncher.h"
@@ -67,7 +68,9 @@ struct Layout {
 
 constexpr int kMaxGroups = 1024;  // workgroups a launch may use (one per CU)
 
-Layout make_layout(const FlashMoeLayerDesc& d) {
+// need_tiled: the tiled variant may run on this workspace (its h rows are
+// reserved per row tile, which costs more than the streaming variant's).
+Layout make_layout(const FlashMoeLayerDesc& d, bool need_tiled) {
   Layout L{};
   const size_t rows = static_cast<size_t>(d.max_tokens) * d.top_k;
   const size_t esz = d.dtype == FLASH_MOE_BF16 ? 2 : 4;
@@ -97,8 +100,9 @@ Layout make_layout(const FlashMoeLayerDesc& d) {
   L.mtiles = take(sizeof(fmoe::TileDesc) * L.max_mtiles);
   // h: [rows, I] routed, or [E, 64, I] when small batches run gate/up densely
   // (the tiled variant reserves 320 rows per row tile, and an expert's last tile is partial)
-  const size_t h_rows = std::max<size_t>({rows, static_cast<size_t>(d.experts) * 64,
-                                          (rows / 256 + static_cast<size_t>(d.experts) + 1) * 320});
+  const size_t h_rows = std::max<size_t>(
+      {rows, static_cast<size_t>(d.experts) * 64,
+       need_tiled ? (rows / 256 + static_cast<size_t>(d.experts) + 1) * 320 : 0});
   L.h = take(esz * h_rows * d.intermediate);
   L.y = take(sizeof(float) * rows * d.hidden);
   const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
@@ -136,6 +140,33 @@ hipError_t validate(const FlashMoeLayerDesc* d) {
   if ((d->flags & ~FLASH_MOE_FLAG_PACK_WEIGHTS) != 0)
     FMOE_FAIL(hipErrorInvalidValue, "unknown flag bits 0x%x", d->flags);
   return hipSuccess;
+}
+
+// The tiled variant needs bf16, tile-aligned shapes and token rows it can
+// address with 32-bit byte offsets. AUTO takes it once an expert sees about 24
+// rows on average when the packed weight copy exists (30B shape, us, streaming /
+// tiled: T=320 283 / 282, T=384 292 / 284, T=512 333 / 289; 235B shape: T=384
+// 920 / 945, T=512 1025 / 960), and from about 3 rows when the weights are read
+// in the caller's row-major layout, which the streaming variant reads poorly
+// (30B: T=32 272 / 270, T=48 296 / 283, T=64 312 / 291, T=128 363 / 297).
+bool tiled_eligible(const FlashMoeLayerDesc& d, int tokens_num) {
+  return d.dtype == FLASH_MOE_BF16 && d.hidden % 256 == 0 && d.intermediate % 128 == 0 &&
+         tokens_num <= fmoe::tiled_max_tokens() &&
+         static_cast<long long>(tokens_num) * d.hidden * 2 < (1ll << 32);
+}
+
+int sched_for(const FlashMoeLayerDesc& d, int tokens_num) {
+  if (d.sched == FLASH_MOE_SCHED_STREAM) return FLASH_MOE_SCHED_STREAM;
+  if (!tiled_eligible(d, tokens_num)) return FLASH_MOE_SCHED_STREAM;
+  if (d.sched == FLASH_MOE_SCHED_TILED) return FLASH_MOE_SCHED_TILED;
+  const long long rows = static_cast<long long>(tokens_num) * d.top_k;
+  const bool packed = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
+  return rows >= (packed ? 24ll : 3ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
+}
+
+// Whether any batch size up to max_tokens may run the tiled variant.
+bool may_run_tiled(const FlashMoeLayerDesc& d) {
+  return d.sched != FLASH_MOE_SCHED_STREAM && tiled_eligible(d, 1);
 }
 
 }  // namespace
@@ -254,7 +285,7 @@ int flashMoeWorkspaceBytes(const FlashMoeLayerDesc* desc, size_t* bytes) {
   const hipError_t v = validate(desc);
   if (v != hipSuccess) return v;
   if (bytes == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null result pointer");
-  *bytes = make_layout(*desc).total;
+  *bytes = make_layout(*desc, may_run_tiled(*desc)).total;
   return hipSuccess;
 }
 
@@ -282,7 +313,7 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
   FlashMoeLauncher* l = new (std::nothrow) FlashMoeLauncher();
   if (l == nullptr) FMOE_FAIL(hipErrorOutOfMemory, "host allocation failed");
   l->desc = *desc;
-  l->layout = make_layout(*desc);
+  l->layout = make_layout(*desc, may_run_tiled(*desc));
 
   auto fail = [&](hipError_t e) {
     if (l->ws) (void)hipFree(l->ws);
@@ -314,28 +345,9 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
   return hipSuccess;
 }
 
-// The tiled variant needs bf16, tile-aligned shapes and token rows it can
-// address with 32-bit byte offsets. AUTO takes it once an expert sees about 24
-// rows on average when the packed weight copy exists (30B shape, us, streaming /
-// tiled: T=320 283 / 282, T=384 292 / 284, T=512 333 / 289; 235B shape: T=384
-// 920 / 945, T=512 1025 / 960), and from about 3 rows when the weights are read
-// in the caller's row-major layout, which the streaming variant reads poorly
-// (30B: T=32 272 / 270, T=48 296 / 283, T=64 312 / 291, T=128 363 / 297).
-static bool tiled_eligible(const FlashMoeLayerDesc& d, int tokens_num) {
-  return d.dtype == FLASH_MOE_BF16 && d.hidden % 256 == 0 && d.intermediate % 128 == 0 &&
-         tokens_num <= fmoe::tiled_max_tokens() &&
-         static_cast<long long>(tokens_num) * d.hidden * 2 < (1ll << 32);
-}
-
 int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num) {
   if (l == nullptr) return -1;
-  const FlashMoeLayerDesc& d = l->desc;
-  if (d.sched == FLASH_MOE_SCHED_STREAM) return FLASH_MOE_SCHED_STREAM;
-  if (!tiled_eligible(d, tokens_num)) return FLASH_MOE_SCHED_STREAM;
-  if (d.sched == FLASH_MOE_SCHED_TILED) return FLASH_MOE_SCHED_TILED;
-  const long long rows = static_cast<long long>(tokens_num) * d.top_k;
-  const bool packed = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
-  return rows >= (packed ? 24ll : 3ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
+  return sched_for(l->desc, tokens_num);
 }
 
 int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int tokens_num,
@@ -355,6 +367,123 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
     FMOE_HIP_CHECK(fmoe::launch_tiled_kernel(p, p.n_groups, stream));
   } else {
     FMOE_HIP_CHECK(fmoe::launch_stream_kernel(p, l->desc.dtype, p.n_groups, stream));
+  }
+  return hipSuccess;
+}
+
+}  // extern "C"
+
+// ------------------------------------------------ the entry point that allocates nothing
+// Workspace of flashMoeLaunchNoAlloc: one array per device, loaded with the
+// code object and held until the process ends. In host code the array's name is
+// only a handle for hipGetSymbolAddress; the device address it yields, kept per
+// device in g_static, is what kernels, fills and copies are given.
+static __device__ __align__(256) unsigned char scratch[FLASH_MOE_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+struct StaticDevice {
+  bool ready = false;
+  unsigned char* ptr = nullptr;  // device address of `scratch` on this device
+  int num_cus = 0;
+  long long ticks_per_ms = 100000;
+};
+StaticDevice g_static[kMaxDevices];
+std::mutex g_static_mutex;
+
+// 16 bytes per thread; n16 = number of 16-byte words to clear
+__global__ void zero_fill_kernel(uint4* dst, size_t n16) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n16) dst[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+// Once per device, with that device current.
+hipError_t static_device(int device, const StaticDevice** out) {
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  StaticDevice& sd = g_static[device];
+  if (!sd.ready) {
+    void* ptr = nullptr;
+    FMOE_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) FMOE_FAIL(hipErrorInvalidSymbol, "no device address for the static workspace");
+    FMOE_HIP_CHECK(hipDeviceGetAttribute(&sd.num_cus, hipDeviceAttributeMultiprocessorCount, device));
+    int khz = 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) == hipSuccess && khz > 0)
+      sd.ticks_per_ms = khz;
+    FMOE_HIP_CHECK(fmoe::prepare_stream_kernel());
+    FMOE_HIP_CHECK(fmoe::prepare_tiled_kernel());
+    sd.ptr = static_cast<unsigned char*>(ptr);
+    sd.ready = true;
+  }
+  *out = &sd;
+  return hipSuccess;
+}
+
+}  // namespace
+
+extern "C" {
+
+int flashMoeLaunchNoAlloc(const FlashMoeLayerDesc* desc, const void* tokens, void* output,
+                          int tokens_num, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const hipError_t v = validate(desc);
+  if (v != hipSuccess) return v;
+  if ((desc->flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0)
+    FMOE_FAIL(hipErrorInvalidValue,
+              "the packed weight copy is weight-sized device memory; flashMoeLaunchNoAlloc has none");
+  if (desc->gate_weights == nullptr || desc->ffn1_weights == nullptr ||
+      desc->ffn2_weights == nullptr)
+    FMOE_FAIL(hipErrorInvalidValue, "null weight pointer");
+  if (tokens_num < 0) FMOE_FAIL(hipErrorInvalidValue, "tokens_num = %i", tokens_num);
+  if (tokens_num > desc->max_tokens)
+    FMOE_FAIL(hipErrorUnknown, "tokens_num = %i exceeds max_tokens = %i", tokens_num,
+              desc->max_tokens);
+  if (tokens_num == 0) return hipSuccess;
+  if (tokens == nullptr || output == nullptr)
+    FMOE_FAIL(hipErrorInvalidValue, "null tokens/output pointer");
+
+  // The workspace is laid out for this call alone: its batch, its variant.
+  FlashMoeLauncher l;
+  l.desc = *desc;
+  l.desc.max_tokens = tokens_num;
+  int sched = sched_for(l.desc, tokens_num);
+  l.layout = make_layout(l.desc, sched == FLASH_MOE_SCHED_TILED);
+  if (sched == FLASH_MOE_SCHED_TILED && desc->sched == FLASH_MOE_SCHED_AUTO &&
+      l.layout.total > static_cast<size_t>(FLASH_MOE_NOALLOC_SCRATCH_BYTES)) {
+    // AUTO: the streaming variant's workspace is smaller, and it serves any batch
+    sched = FLASH_MOE_SCHED_STREAM;
+    l.desc.sched = FLASH_MOE_SCHED_STREAM;
+    l.layout = make_layout(l.desc, false);
+  }
+  if (l.layout.total > static_cast<size_t>(FLASH_MOE_NOALLOC_SCRATCH_BYTES))
+    FMOE_FAIL(hipErrorUnknown,
+              "%i tokens of this layer need %zu bytes of workspace; the static one holds %zu "
+              "(use flashMoeCreate / flashMoeLaunch for this size)",
+              tokens_num, l.layout.total, static_cast<size_t>(FLASH_MOE_NOALLOC_SCRATCH_BYTES));
+  int device = 0;
+  FMOE_HIP_CHECK(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) FMOE_FAIL(hipErrorInvalidDevice, "device %i", device);
+  const StaticDevice* sd = nullptr;
+  const hipError_t se = static_device(device, &sd);
+  if (se != hipSuccess) return se;
+  l.ws = reinterpret_cast<char*>(sd->ptr);
+  l.device = device;
+  l.num_cus = sd->num_cus;
+  l.ticks_per_ms = sd->ticks_per_ms;
+  l.spin_limit = 2000 * sd->ticks_per_ms;
+
+  // The array keeps what the last call (of any shape) left in it: counters, flags
+  // and masks of this call's layout must start at zero. A kernel, not a memset,
+  // so that the call can be recorded into a HIP graph.
+  const size_t n16 = (l.layout.zero_bytes + 15) / 16;
+  hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>((n16 + 255) / 256)), dim3(256), 0,
+                     stream, reinterpret_cast<uint4*>(sd->ptr), n16);
+  FMOE_HIP_CHECK(hipGetLastError());
+  const fmoe::Params p = make_params(&l, tokens, output, tokens_num);
+  if (sched == FLASH_MOE_SCHED_TILED) {
+    FMOE_HIP_CHECK(fmoe::launch_tiled_kernel(p, p.n_groups, stream));
+  } else {
+    FMOE_HIP_CHECK(fmoe::launch_stream_kernel(p, desc->dtype, p.n_groups, stream));
   }
   return hipSuccess;
 }

@@ -87,6 +87,30 @@ int flashMoeRefreshWeights(FlashMoeLauncher* l, void* stream);
 int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int tokens_num,
                    void* stream);
 
+/* One forward pass that allocates nothing: for callers that cannot call
+ * hipMalloc (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it). It has no counterpart in the reference, whose launcher allocates
+ * its buffers in Init (src/hip/launcher/moeKernelLauncher.hip:147-165). Same
+ * kernels and results as flashMoeCreate + flashMoeLaunch on the same inputs, but
+ * the workspace is a static device array of FLASH_MOE_NOALLOC_SCRATCH_BYTES that
+ * every device the library runs on holds until the process ends. `desc` is read
+ * as in flashMoeCreate (weights borrowed for the duration of the launch; flags
+ * must be 0: there is no packed weight copy); the workspace is laid out for
+ * tokens_num alone, and with FLASH_MOE_SCHED_AUTO the variant is the one
+ * flashMoeLaunch would take if its workspace fits, else the streaming one.
+ * hipErrorUnknown when tokens_num > desc->max_tokens or when that batch needs
+ * more workspace than the array holds (it holds about 700 tokens of the
+ * E128/H2048/I768/top-8 bf16 shape and 300 of E128/H4096/I1536/top-8 with the
+ * streaming variant); nothing is enqueued then.
+ * Enqueues a small clearing kernel and the layer's kernel on `stream`, waits
+ * for nothing, calls no hipMalloc/hipFree. The first call on a device looks up
+ * the array's address and the device's properties (make it outside a graph
+ * capture). All calls on a device share the one array: calls that may overlap
+ * on a device (two streams, two threads) race; order them on one stream. */
+#define FLASH_MOE_NOALLOC_SCRATCH_BYTES (64u << 20)
+int flashMoeLaunchNoAlloc(const FlashMoeLayerDesc* desc, const void* tokens, void* output,
+                          int tokens_num, void* stream);
+
 /* Frees the workspace; synchronises `stream`. */
 int flashMoeDestroy(FlashMoeLauncher* l, void* stream);
 
