@@ -68,8 +68,7 @@ struct Layout {
 
 constexpr int kMaxGroups = 1024;  // workgroups a launch may use (one per CU)
 
-// need_tiled: the tiled variant may run on this workspace (its h rows are
-// reserved per row tile, which costs more than the streaming variant's).
+// need_tiled: the tiled variant may run on this workspace.
 Layout make_layout(const FlashMoeLayerDesc& d, bool need_tiled) {
   Layout L{};
   const size_t rows = static_cast<size_t>(d.max_tokens) * d.top_k;
@@ -99,10 +98,8 @@ Layout make_layout(const FlashMoeLayerDesc& d, bool need_tiled) {
   L.row_w = take(sizeof(float) * rows);
   L.mtiles = take(sizeof(fmoe::TileDesc) * L.max_mtiles);
   // h: [rows, I] routed, or [E, 64, I] when small batches run gate/up densely
-  // (the tiled variant reserves 320 rows per row tile, and an expert's last tile is partial)
-  const size_t h_rows = std::max<size_t>(
-      {rows, static_cast<size_t>(d.experts) * 64,
-       need_tiled ? (rows / 256 + static_cast<size_t>(d.experts) + 1) * 320 : 0});
+  (void)need_tiled;  // both variants keep h as [rows, I]
+  const size_t h_rows = std::max<size_t>(rows, static_cast<size_t>(d.experts) * 64);
   L.h = take(esz * h_rows * d.intermediate);
   L.y = take(sizeof(float) * rows * d.hidden);
   const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;

@@ -1,25 +1,27 @@
-// Persistent MoE kernel, tiled ("fat") variant for gfx950: the shape for
-// batches where an expert sees hundreds of rows (prefill) and the layer is
-// bound by MFMA throughput, bf16 only.
+// Persistent MoE kernel, tiled variant for gfx950: the shape for batches where an
+// expert sees many rows (prefill) and the layer is bound by matrix throughput,
+// bf16 only.
 //
-// One workgroup of 8 waves per CU (two per SIMD) draws workgroup-wide task
-// tickets from the same kind of counter as the streaming variant; tasks depend
-// only on tasks with smaller tickets. Stages (ticket order):
-//   router   32 tokens x all experts: logits in the oracle's summation order
-//            as a chain of f32 matrix instructions (four waves multiply, four
-//            waves load through LDS), then top-k / softmax
+// One workgroup of 4 waves per CU (one per SIMD, each with the SIMD's whole
+// register file) draws workgroup-wide task tickets from the same kind of counter
+// as the streaming variant; tasks depend only on tasks with smaller tickets.
+// Stages (ticket order):
+//   router   16 tokens x all experts: logits in the oracle's summation order as
+//            chains of f32 matrix instructions, then top-k / softmax
 //   scan     one wave per expert: counts and running prefixes of its mask
-//            words; then one short task: offsets and the 256-row tile table
+//            words; then one short task: offsets and the row-tile table
 //   scatter  32 tokens: permuted row of every (token, slot)
-//   gate/up  (row tile, 128 h columns): 256x256 MFMA tile, gate and up
-//            columns side by side so that SiLU(gate)*up happens in registers
+//   gate/up  (row tile, 128 h columns): 256 token rows x 256 weight rows, gate
+//            and up rows side by side so that SiLU(gate)*up happens in registers
 //   down     (row tile, 256 output columns): same tile, weighted bf16 rows to y
 //   combine  8 tokens: out = sum over slots of y
-// GEMM tile: 256 token rows x 256 weight rows, K stepped by 32 through four LDS
-// stages that are filled straight from global memory; each wave owns 128
-// weight rows x 64 token rows of it as 4x2 MFMA 32x32x16 blocks, 128
-// accumulator registers. Weight rows are the MFMA "A" operand so that a lane
-// ends up with runs of 4 consecutive output columns of one token row.
+// GEMM tile: up to 256 token rows x 256 weight rows, K stepped by 64 through two
+// LDS stages that are filled straight from global memory in whole 128-byte
+// lines; each wave owns 64 weight rows x all token rows of it as 2x8 MFMA
+// 32x32x16 blocks, 256 accumulator registers. Weight rows are the MFMA "A"
+// operand so that a lane ends up with runs of 4 consecutive output columns of
+// one token row. A tile with fewer rows multiplies fewer token blocks, so its
+// time follows its rows.
 //
 // Replaces, for this regime, the reference's moeKernel
 // (src/hip/kernel/moeKernel.h:37-107) and its TILE_M=1 GEMV tiles
@@ -33,30 +35,18 @@ namespace fmoe {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int TM = 256;            // token rows per tile
-constexpr int TN = 256;            // weight rows per tile
-constexpr int TK = 32;             // k per LDS stage (one 64-byte row slice)
-constexpr int STAGES = 4;          // LDS stages in flight
-constexpr int STAGE_BYTES = (TM + TN) * TK * 2;  // 32 KiB: weight rows, then token rows
-constexpr int T_THREADS = 512;
-constexpr int WAVES = T_THREADS / 64;  // two per SIMD: one wave's loads and LDS reads hide behind the other's MFMAs
-constexpr int WJ = 16 / WAVES;         // 32-row token blocks per wave (each wave: 128 weight rows x 32*WJ token rows)
-constexpr int LQ = 16 / WAVES;         // 16-row loads per operand, stage and wave
-constexpr int G1_COLS = TN / 2;    // h columns per gate/up task
-constexpr int RT_TOK = 32;         // tokens per router / scatter task
-constexpr int CMB_TOK = 8;         // tokens per combine task
 
-constexpr int TILE_LDS_BYTES = STAGES * STAGE_BYTES;  // 131072
-constexpr int ROUTER_LDS_BYTES = 4 * 24576 + RT_TOK * MAX_EXPERTS * 4 + WAVES * MAX_TOPK * 8;
-// Tall row tiles: an expert's last 1..TALL_EXTRA rows join its last full tile instead of
-// costing a pass of their own over the expert's weights.
-constexpr int TALL_EXTRA = 64;
-constexpr int TALL_TM = TM + TALL_EXTRA;                       // 320 token rows
-constexpr int TALL_STAGE_BYTES = (TN + TALL_TM) * TK * 2;      // 36 KiB: weight rows, then token rows
-constexpr int TALL_LDS_BYTES = STAGES * TALL_STAGE_BYTES;      // 147456
-constexpr int HT_ROWS = TALL_TM;                               // rows a row tile owns in h
-constexpr int TILED_LDS_BYTES_0 = TILE_LDS_BYTES > ROUTER_LDS_BYTES ? TILE_LDS_BYTES : ROUTER_LDS_BYTES;
-constexpr int TILED_LDS_BYTES = TILED_LDS_BYTES_0 > TALL_LDS_BYTES ? TILED_LDS_BYTES_0 : TALL_LDS_BYTES;
+constexpr int JT_MAX = 10;         // 32-row token blocks of the tallest row tile
+constexpr int TM_MAX = 32 * JT_MAX;  // 320 token rows
+constexpr int TN = 256;            // weight rows per tile
+constexpr int KS = 64;             // k per LDS stage
+constexpr int ROWB = KS * 2;       // bytes of a row per stage: one 128-byte line
+constexpr int T_THREADS = 256;
+constexpr int WAVES = T_THREADS / 64;  // one per SIMD
+constexpr int NLD = 8;             // 8-row loads per wave, operand and stage
+constexpr int G1_COLS = TN / 2;    // h columns per gate/up task
+constexpr int RT_TOK = 32;         // tokens per scatter task
+constexpr int CMB_TOK = 8;         // tokens per combine task
 
 extern __shared__ __align__(16) unsigned char lds_raw[];
 
@@ -194,189 +184,29 @@ __device__ __forceinline__ void load_to_lds(unsigned off, const unsigned char* b
 // --------------------------------------------------------------------- router
 // Logits as in test/singleGPU/cpp/moe/reference/refGemm.h:21-24: one chain per
 // output, k ascending, one rounding per step. The chain runs on the matrix
-// core: V_MFMA_F32_32X32X2_F32 adds its two products to the accumulator one
-// after the other in k order (checked bit for bit against a CPU fmaf chain; so
-// do 16X16X1 and 16X16X4), and a product of two bf16 values is exact in float,
-// so every step is the oracle's acc = fmaf(x, w, acc). A dependent chain of
-// these instructions runs at the matrix core's full rate (64 cycles each).
-// Waves 0..3 carry 32 tokens x 32 experts each, one wave per SIMD; waves 4..7
-// are the loaders: they bring the 32 token rows and
-// 128 expert rows in, 64 k at a time, with coalesced direct-to-LDS loads, four
-// stages deep. Stage rows are 144 bytes (128 of data, 16 of padding), so the
-// 16-byte reads of 16 rows at one k fall into different banks and every read
-// address is a per-lane base plus an immediate. (One LDS read costs a wave
-// about 22 cycles of issue whatever its width, hence 16-byte reads.)
+// core: V_MFMA_F32_16X16X4_F32 adds its four products to the accumulator one
+// after the other in k order (checked bit for bit against a CPU fmaf chain), and
+// a product of two bf16 values is exact in float, so every step is the oracle's
+// acc = fmaf(x, w, acc). A dependent chain of these instructions runs at the
+// matrix core's full rate, so one chain per SIMD would do; a wave carries two
+// (16 tokens x experts 16w..16w+15 and 64+16w..64+16w+15 of a slab of 128), which
+// is what four waves need to cover the slab.
+// All waves load: 64 k of the 16 token rows and the 128 expert rows per stage,
+// four stages deep, with coalesced direct-to-LDS loads. Stage rows are 144 bytes
+// (128 of data, 16 of padding), so the 16-byte reads of 16 rows at one k fall
+// into different banks. Lane l multiplies row l % 16 of both operands at
+// k = 4*s + l/16: of the eight bf16 a 16-byte read brings, elements l/16 and
+// 4 + l/16, each moved into the upper half of a zero word by one byte permute.
 // Then selection as in refTopk.h:36-58 / refMoeGate.h:27-30.
-constexpr int RT_ROW_BYTES = 144;
-constexpr int RT_LOADS = 6;                       // loads per loader wave and stage
-constexpr int RT_STAGE_BYTES = 4 * RT_LOADS * 1024;  // 24 KiB
-constexpr int RT_TOK_LOADS = (RT_TOK * 9 + 63) / 64; // loads that hold token rows
-constexpr int RT_EXP_BASE = RT_TOK_LOADS * 1024;     // byte offset of the expert rows in a stage
-constexpr int RT_STAGES = 4;
-static_assert(RT_EXP_BASE + 128 * RT_ROW_BYTES <= RT_STAGE_BYTES, "router stage too small");
-
-__device__ __noinline__ void tiled_router_task(ParamsRef pv, int blk) {
-  ParamsRef p = uniform_params(pv);
-  const int T = uni(p.T), E = uni(p.E), H = uni(p.H);
-  const unsigned char* tokens = uni(reinterpret_cast<const unsigned char*>(p.tokens));
-  const unsigned char* gate = uni(reinterpret_cast<const unsigned char*>(p.gate));
-  const float* bias = uni(p.bias);
-  unsigned* keys = reinterpret_cast<unsigned*>(lds_raw + RT_STAGES * RT_STAGE_BYTES);  // [RT_TOK][MAX_EXPERTS] ordered logits
-  double* sel = reinterpret_cast<double*>(keys + RT_TOK * MAX_EXPERTS);  // WAVES x MAX_TOPK
-  const unsigned lds_addr = uni(static_cast<unsigned>(
-      reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
-  const int tid = threadIdx.x;
-  const int wave = uni(tid >> 6), lane = tid & 63;
-  const bool loader = wave >= 4;
-  const int t0 = uni(blk) * RT_TOK;
-  const int nsteps = H >> 6;
-
-  for (int e0 = 0; e0 < E; e0 += 128) {
-    // loader: load ld = 6*w + i fills the 64 16-byte slots from slot 64*ld on. Loads
-    // 0..4 hold the token rows, loads 5..23 the expert rows (from byte RT_EXP_BASE);
-    // within a region slot g is position g % 9 of row g / 9 (position 8 is padding,
-    // slots past the last row repeat it).
-    unsigned goff[RT_LOADS];
-#pragma unroll
-    for (int i = 0; i < RT_LOADS; ++i) {
-      const int ld = (wave & 3) * RT_LOADS + i;  // uniform
-      const bool tok = ld < RT_TOK_LOADS;
-      const int g = (tok ? ld : ld - RT_TOK_LOADS) * 64 + lane;
-      const int row = min(g / 9, (tok ? RT_TOK : 128) - 1);
-      const int pos = min(g % 9, 7);
-      const int grow = tok ? min(t0 + row, T - 1) : min(e0 + row, E - 1);
-      goff[i] = static_cast<unsigned>(grow) * static_cast<unsigned>(H * 2) + pos * 16;
-    }
-    auto issue = [&](int step) {
-      const int src = min(step, nsteps - 1);  // past the end: refill with the last step (never read)
-      const unsigned st = lds_addr + (step & (RT_STAGES - 1)) * RT_STAGE_BYTES +
-                          ((wave & 3) * RT_LOADS) * 1024;
-#pragma unroll
-      for (int i = 0; i < RT_LOADS; ++i) {
-        const bool tok = (wave & 3) * RT_LOADS + i < RT_TOK_LOADS;
-        load_to_lds(goff[i], (tok ? tokens : gate) + static_cast<size_t>(src) * 128, st + i * 1024);
-      }
-    };
-    // consumer: wave w multiplies the 32 token rows with expert rows 32*w .. 32*w+31.
-    // Lane l: row l % 32 of both; V_MFMA_F32_32X32X2_F32 takes k = 2*s + l/32 from it,
-    // i.e. the low or the high half of 32-bit word s of the row: the byte permute
-    // moves that half into the upper 16 bits of a zero word, which makes the float.
-    const int r32 = lane & 31, kh = lane >> 5;
-    const unsigned pick = kh ? 0x07060C0Cu : 0x05040C0Cu;
-    const unsigned char* xptr = lds_raw + r32 * RT_ROW_BYTES;
-    const unsigned char* wptr = lds_raw + RT_EXP_BASE + ((wave & 3) * 32 + r32) * RT_ROW_BYTES;
-    f32x16 acc;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-
-    // Operands of half a stage: four 16-byte chunks (8 k each) of both rows.
-    struct Half {
-      uint4 a[4], w[4];
-    };
-    auto read_half = [&](Half& h, int stage, int hf) {
-      const int so = (stage & (RT_STAGES - 1)) * RT_STAGE_BYTES + hf * 64;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        h.a[c] = *reinterpret_cast<const uint4*>(xptr + so + c * 16);
-        h.w[c] = *reinterpret_cast<const uint4*>(wptr + so + c * 16);
-      }
-    };
-    // The 16 MFMAs of one half, and between them the reads of another half: one pair
-    // of reads after every fourth MFMA. A read costs the wave about 20 cycles of
-    // issue, which fits in the 64 cycles the next (dependent) MFMA has to wait anyway;
-    // the scheduling barriers keep the compiler from moving the reads to the end.
-    auto chain_and_read = [&](const Half& h, Half& nx, int stage, int hf) {
-      const int so = (stage & (RT_STAGES - 1)) * RT_STAGE_BYTES + hf * 64;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const unsigned xw[4] = {h.a[c].x, h.a[c].y, h.a[c].z, h.a[c].w};
-        const unsigned ww[4] = {h.w[c].x, h.w[c].y, h.w[c].z, h.w[c].w};
-#pragma unroll
-        for (int m = 0; m < 4; ++m)
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(
-              __uint_as_float(__builtin_amdgcn_perm(xw[m], 0u, pick)),
-              __uint_as_float(__builtin_amdgcn_perm(ww[m], 0u, pick)), acc, 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        nx.a[c] = *reinterpret_cast<const uint4*>(xptr + so + c * 16);
-        nx.w[c] = *reinterpret_cast<const uint4*>(wptr + so + c * 16);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    };
-
-    // Loaders and consumers run separate loops with the same number of barriers:
-    // barrier s (in the middle of step s) means "stage s+1 is in, nobody reads
-    // stage s any more".
-    if (loader) {
-      issue(0);
-      issue(1);
-      issue(2);
-      issue(3);
-      wait_vm<3 * RT_LOADS>();
-      __builtin_amdgcn_s_barrier();  // stage 0 is in
-      for (int s = 0; s < nsteps; ++s) {
-        wait_vm<2 * RT_LOADS>();  // stage s+1 is in; s+2 and s+3 may be in flight
-        __builtin_amdgcn_s_barrier();
-        issue(s + RT_STAGES);     // into the stage every consumer has just left
-      }
-    } else {
-      Half h0, h1;
-      __builtin_amdgcn_s_barrier();  // stage 0 is in
-      asm volatile("" ::: "memory");
-      read_half(h0, 0, 0);
-      for (int s = 0; s < nsteps; ++s) {
-        chain_and_read(h0, h1, s, 1);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave no longer reads stage s
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        // past the last stage this reads the stage the loaders refilled with the last
-        // step's data again; the values are never used
-        chain_and_read(h1, h0, s + 1, 0);
-      }
-    }
-    if (loader) wait_vm<0>();       // nothing may land in a stage after this slab
-    __builtin_amdgcn_s_barrier();   // the stages may be refilled for the next slab
-    asm volatile("" ::: "memory");
-    if (!loader) {
-      // acc[r] of lane l: token 8*(r/4) + 4*(l/32) + r%4, expert e0 + 32*w + l%32
-      const int e = e0 + (wave & 3) * 32 + r32;
-      const float bv = (bias != nullptr && e < E) ? as_global(bias)[e] : 0.0f;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float v = acc[r];
-        if (bias != nullptr) v = __fadd_rn(v, bv);
-        if (e < MAX_EXPERTS)
-          keys[(8 * (r >> 2) + 4 * kh + (r & 3)) * MAX_EXPERTS + e] = ordered_bits(v, e < E);
-      }
-    }
-  }
-  __syncthreads();
-  // selection: the tokens are dealt out over all waves
-  double* lex = sel + wave * MAX_TOPK;
-  for (int i = 0; i < RT_TOK / WAVES; ++i) {
-    const int tl = wave * (RT_TOK / WAVES) + i;
-    const int t = t0 + tl;
-    if (t < T) {
-      unsigned val[MAX_EXPERTS / 64];
-#pragma unroll
-      for (int j = 0; j < MAX_EXPERTS / 64; ++j) {
-        const int e = lane + 64 * j;
-        val[j] = e < E ? keys[tl * MAX_EXPERTS + e] : 0u;
-      }
-      router_select_max(p, t, val, lex);
-    }
-  }
-}
-
-// The same for 16 tokens, used while that still gives every workgroup at most one
-// router task (T <= 16 x workgroups): with 32-token tasks half of the CUs or more
-// would sit through the router idle. The chains run on V_MFMA_F32_16X16X4_F32
-// (which also adds its products in k order, one rounding each): wave w carries
-// the 16 tokens x experts 16w..16w+15 of the slab. All eight waves load: 64 k of
-// the 16 token rows and the 128 expert rows per stage, rows 144 bytes apart as
-// above. Lane l multiplies row l % 16 of both operands at k = 4*s + l/16: of the
-// eight bf16 a 16-byte read brings, elements l/16 and 4 + l/16, each moved into
-// the upper half of a zero word by one byte permute.
 constexpr int RT16_TOK = 16;
+constexpr int RT_ROW_BYTES = 144;
+constexpr int RT_STAGES = 4;
+constexpr int RT_NL = 6;                                  // loads per wave and stage
+constexpr int RT_STAGE_BYTES = WAVES * RT_NL * 1024;      // 24 KiB
+constexpr int RT_NROWS = RT16_TOK + 128;
+static_assert(RT_NROWS * 9 <= WAVES * RT_NL * 64, "router stage too small");
+constexpr int ROUTER_LDS_BYTES = RT_STAGES * RT_STAGE_BYTES + RT16_TOK * MAX_EXPERTS * 4 + WAVES * MAX_TOPK * 8;
+
 __device__ __forceinline__ void load_to_lds_addr(const unsigned char* addr, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
@@ -384,14 +214,14 @@ __device__ __forceinline__ void load_to_lds_addr(const unsigned char* addr, unsi
                : "memory");
 }
 
-__device__ __noinline__ void tiled_router16_task(ParamsRef pv, int blk) {
+__device__ __noinline__ void tiled_router_task(ParamsRef pv, int blk) {
   ParamsRef p = uniform_params(pv);
   const int T = uni(p.T), E = uni(p.E), H = uni(p.H);
   const unsigned char* tokens = uni(reinterpret_cast<const unsigned char*>(p.tokens));
   const unsigned char* gate = uni(reinterpret_cast<const unsigned char*>(p.gate));
   const float* bias = uni(p.bias);
   unsigned* keys = reinterpret_cast<unsigned*>(lds_raw + RT_STAGES * RT_STAGE_BYTES);  // [RT16_TOK][MAX_EXPERTS]
-  double* sel = reinterpret_cast<double*>(keys + RT_TOK * MAX_EXPERTS);                // WAVES x MAX_TOPK
+  double* sel = reinterpret_cast<double*>(keys + RT16_TOK * MAX_EXPERTS);              // WAVES x MAX_TOPK
   const unsigned lds_addr = uni(static_cast<unsigned>(
       reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
   const int tid = threadIdx.x;
@@ -400,19 +230,17 @@ __device__ __noinline__ void tiled_router16_task(ParamsRef pv, int blk) {
   const int nsteps = H >> 6;
   // slot g of a stage (16 bytes): position g % 9 of row g / 9 (position 8 is padding);
   // rows 0..15 are the tokens, 16..143 the experts of the slab; slots past the last row repeat it
-  constexpr int NL = 3;  // loads per wave and stage: 1536 slots >= 144 rows x 9
-  constexpr int NROWS = RT16_TOK + 128;
-  static_assert(NROWS * 9 <= WAVES * NL * 64 && WAVES * NL * 1024 == RT_STAGE_BYTES, "router stage");
   const int r16 = lane & 15, kq = lane >> 4;
   const unsigned pick = kq == 0 ? 0x01000C0Cu : kq == 1 ? 0x03020C0Cu : kq == 2 ? 0x05040C0Cu : 0x07060C0Cu;
   const int xoff = r16 * RT_ROW_BYTES;
-  const int woff = (RT16_TOK + 16 * wave + r16) * RT_ROW_BYTES;
+  const int woff0 = (RT16_TOK + 16 * wave + r16) * RT_ROW_BYTES;
+  const int woff1 = (RT16_TOK + 64 + 16 * wave + r16) * RT_ROW_BYTES;
   for (int e0 = 0; e0 < E; e0 += 128) {
-    const unsigned char* src[NL];
+    const unsigned char* src[RT_NL];
 #pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const int g = (wave * NL + i) * 64 + lane;
-      const int row = min(g / 9, NROWS - 1);
+    for (int i = 0; i < RT_NL; ++i) {
+      const int g = (wave * RT_NL + i) * 64 + lane;
+      const int row = min(g / 9, RT_NROWS - 1);
       const int pos = min(g % 9, 7);
       const unsigned char* base =
           row < RT16_TOK ? tokens + static_cast<size_t>(min(t0 + row, T - 1)) * H * 2
@@ -421,31 +249,36 @@ __device__ __noinline__ void tiled_router16_task(ParamsRef pv, int blk) {
     }
     auto issue = [&](int step) {  // past the last step: the last one again, into a stage nobody reads
       const size_t koff = static_cast<size_t>(min(step, nsteps - 1)) * 128;
-      const unsigned st = lds_addr + (step & (RT_STAGES - 1)) * RT_STAGE_BYTES + wave * (NL * 1024);
+      const unsigned st = lds_addr + (step & (RT_STAGES - 1)) * RT_STAGE_BYTES + wave * (RT_NL * 1024);
 #pragma unroll
-      for (int i = 0; i < NL; ++i) load_to_lds_addr(src[i] + koff, st + i * 1024);
+      for (int i = 0; i < RT_NL; ++i) load_to_lds_addr(src[i] + koff, st + i * 1024);
     };
-    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-    // Operands of half a stage (32 k): four 16-byte chunks of both rows. While the 8
-    // matrix instructions of one half run, the next half is read, one chunk of both
-    // rows after each pair; the scheduling barriers keep the reads from being
-    // gathered in front of their first use, where their latency would be exposed.
+    f32x4 acc0 = f32x4{0.f, 0.f, 0.f, 0.f}, acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
+    // Operands of half a stage (32 k): four 16-byte chunks of the token row and of the
+    // two expert rows. While the 16 matrix instructions of one half run, the next half is
+    // read, one chunk of the three rows after each four; the scheduling barriers keep the
+    // reads from being gathered in front of their first use.
     struct Half {
-      uint4 a[4], w[4];
+      uint4 a[4], w0[4], w1[4];
     };
     auto read_chunk = [&](Half& h, const unsigned char* hb, int c4) {
       h.a[c4] = *reinterpret_cast<const uint4*>(hb + xoff + 16 * c4);
-      h.w[c4] = *reinterpret_cast<const uint4*>(hb + woff + 16 * c4);
+      h.w0[c4] = *reinterpret_cast<const uint4*>(hb + woff0 + 16 * c4);
+      h.w1[c4] = *reinterpret_cast<const uint4*>(hb + woff1 + 16 * c4);
     };
     auto chain_and_read = [&](const Half& h, Half& nx, const unsigned char* nb) {
 #pragma unroll
       for (int c4 = 0; c4 < 4; ++c4) {
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
-            __uint_as_float(__builtin_amdgcn_perm(h.a[c4].y, h.a[c4].x, pick)),
-            __uint_as_float(__builtin_amdgcn_perm(h.w[c4].y, h.w[c4].x, pick)), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
-            __uint_as_float(__builtin_amdgcn_perm(h.a[c4].w, h.a[c4].z, pick)),
-            __uint_as_float(__builtin_amdgcn_perm(h.w[c4].w, h.w[c4].z, pick)), acc, 0, 0, 0);
+        const float xl = __uint_as_float(__builtin_amdgcn_perm(h.a[c4].y, h.a[c4].x, pick));
+        const float xh = __uint_as_float(__builtin_amdgcn_perm(h.a[c4].w, h.a[c4].z, pick));
+        acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(
+            xl, __uint_as_float(__builtin_amdgcn_perm(h.w0[c4].y, h.w0[c4].x, pick)), acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(
+            xl, __uint_as_float(__builtin_amdgcn_perm(h.w1[c4].y, h.w1[c4].x, pick)), acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(
+            xh, __uint_as_float(__builtin_amdgcn_perm(h.w0[c4].w, h.w0[c4].z, pick)), acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(
+            xh, __uint_as_float(__builtin_amdgcn_perm(h.w1[c4].w, h.w1[c4].z, pick)), acc1, 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         read_chunk(nx, nb, c4);
         __builtin_amdgcn_sched_barrier(0);
@@ -453,7 +286,7 @@ __device__ __noinline__ void tiled_router16_task(ParamsRef pv, int blk) {
     };
 #pragma unroll
     for (int st = 0; st < RT_STAGES; ++st) issue(st);
-    wait_vm<(RT_STAGES - 1) * NL>();
+    wait_vm<(RT_STAGES - 1) * RT_NL>();
     __builtin_amdgcn_s_barrier();  // stage 0 is in
     asm volatile("" ::: "memory");
     Half h0, h1;
@@ -462,7 +295,7 @@ __device__ __noinline__ void tiled_router16_task(ParamsRef pv, int blk) {
     for (int st = 0; st < nsteps; ++st) {
       chain_and_read(h0, h1, lds_raw + (st & (RT_STAGES - 1)) * RT_STAGE_BYTES + 64);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave no longer reads stage st
-      wait_vm<(RT_STAGES - 2) * NL>();                    // its loads of stage st+1 are in
+      wait_vm<(RT_STAGES - 2) * RT_NL>();                 // its loads of stage st+1 are in
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
       issue(st + RT_STAGES);
@@ -472,18 +305,23 @@ __device__ __noinline__ void tiled_router16_task(ParamsRef pv, int blk) {
     wait_vm<0>();                  // nothing may land in a stage after this slab
     __builtin_amdgcn_s_barrier();  // the stages may be refilled for the next slab
     asm volatile("" ::: "memory");
-    // acc[v] of lane l: token 4*(l/16) + v, expert e0 + 16*wave + l%16
-    const int e = e0 + 16 * wave + r16;
-    const float bv = (bias != nullptr && e < E) ? as_global(bias)[e] : 0.0f;
+    // acc[v] of lane l: token 4*(l/16) + v, expert e0 + (0 | 64) + 16*wave + l%16
+    const int ea = e0 + 16 * wave + r16, eb = ea + 64;
+    const float bva = (bias != nullptr && ea < E) ? as_global(bias)[ea] : 0.0f;
+    const float bvb = (bias != nullptr && eb < E) ? as_global(bias)[eb] : 0.0f;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      float x = acc[v];
-      if (bias != nullptr) x = __fadd_rn(x, bv);
-      if (e < MAX_EXPERTS) keys[(4 * kq + v) * MAX_EXPERTS + e] = ordered_bits(x, e < E);
+      float xa = acc0[v], xb = acc1[v];
+      if (bias != nullptr) {
+        xa = __fadd_rn(xa, bva);
+        xb = __fadd_rn(xb, bvb);
+      }
+      if (ea < MAX_EXPERTS) keys[(4 * kq + v) * MAX_EXPERTS + ea] = ordered_bits(xa, ea < E);
+      if (eb < MAX_EXPERTS) keys[(4 * kq + v) * MAX_EXPERTS + eb] = ordered_bits(xb, eb < E);
     }
   }
   __syncthreads();
-  // selection: two tokens per wave
+  // selection: four tokens per wave
   double* lex = sel + wave * MAX_TOPK;
   for (int i = 0; i < RT16_TOK / WAVES; ++i) {
     const int tl = wave * (RT16_TOK / WAVES) + i;
@@ -500,11 +338,13 @@ __device__ __noinline__ void tiled_router16_task(ParamsRef pv, int blk) {
   }
 }
 
+
 // ----------------------------------------------------------------------- scan
 // Same tables as the streaming variant's scan, in two steps. Expert scan: one
 // wave per expert walks the expert's mask words 64 at a time and writes the
 // running count in front of every word (word_prefix) and the expert's total.
-// Final scan: one wave turns the totals into row offsets and the row-tile table.
+// Final scan: one wave turns the totals into row offsets and the row-tile table
+// (an expert's rows in as few tiles of at most TM_MAX rows as possible, of equal size).
 constexpr int SCAN_EXPERTS = T_THREADS / 64;  // experts per expert-scan task
 
 __device__ __noinline__ void tiled_expert_scan_task(ParamsRef pv, int blk) {
@@ -541,11 +381,9 @@ __device__ __noinline__ void tiled_scan_task(ParamsRef pv) {
       const int c = e < r.E ? ldc(&r.expert_count[e]) : 0;
       const int incl = wave_inclusive_scan(c);
       const int off = base + incl - c;
-      // Tiles of up to TALL_TM rows where that saves passes over the expert's weights
-      // (a tall tile costs about an eighth more than one of TM rows): tiles keep TM
-      // rows as long as the rest still fits the remaining tiles at TALL_TM each.
-      const int nt_norm = (c + TM - 1) / TM, nt_tall = (c + TALL_TM - 1) / TALL_TM;
-      const int nt = nt_tall * 9 < nt_norm * 8 ? nt_tall : nt_norm;
+      // balanced tiles of at most TM_MAX rows, whole 32-row blocks
+      const int nt = (c + TM_MAX - 1) / TM_MAX;
+      const int per = nt > 0 ? ((c + nt - 1) / nt + 31) / 32 * 32 : 0;
       const int tincl = wave_inclusive_scan(nt);
       const int toff = tile_base + tincl - nt;
       if (e < r.E) {
@@ -553,7 +391,7 @@ __device__ __noinline__ void tiled_scan_task(ParamsRef pv) {
         int done = 0;
         for (int i = 0; i < nt; ++i) {
           const int left = c - done;
-          const int tr = max(min(TM, left), left - TALL_TM * (nt - 1 - i));
+          const int tr = min(per, left);
           if (toff + i < r.max_mtiles) {
             stc16(&r.mtiles[toff + i],
                   make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + done),
@@ -587,636 +425,345 @@ __device__ void tiled_scatter_task(ParamsRef p, int blk) {
 }
 
 // -------------------------------------------------------------- the GEMM tile
-// Operands go HBM/L2 -> LDS directly (global_load_lds_dwordx4: lane l's 16
-// bytes land at LDS base + 16*l, from any global address), four stages of 32
-// k deep, so no register staging, no LDS write instructions and almost no VALU
-// work in the loop. A wave issues in order: every LDS read (about 20 cycles)
-// and every direct-to-LDS load it issues delays its own next MFMA, which is
-// why two waves share a SIMD here: one multiplies while the other issues.
+// Operands go HBM/L2 -> LDS directly (global_load_lds_dwordx4: lane l's 16 bytes
+// land at LDS base + 16*l, from any global address), in stages of 64 k: one
+// 128-byte line of every operand row, so every request uses whole cache lines
+// whatever the row pitch. Two stages; no register staging, no LDS write
+// instructions, almost no vector-ALU work in the loop.
 //
-// LDS stage layout: rows of 64 bytes (32 bf16), unpadded, weight rows 0..255
-// then token rows 0..255. Row R keeps its four 16-byte chunks permuted: chunk C
-// sits at position C ^ ((R >> 2) & 3), so the 16 rows a quarter-wave reads
-// together (256 bytes, all 64 banks) fall in 16 different 16-byte bank groups.
-// One wave-wide load fills 16 rows; lane l loads the chunk that belongs at
-// position l & 3 of row l >> 2.
-// Weights come either from the caller's row-major matrices (64 bytes of each of
-// 16 rows per load) or, when the launcher keeps the packed copy, from that: the
-// streaming variant's layout holds every 16-row block of a k-step as one
-// contiguous 1 KiB run [chunk 0..3][row 0..15][16 B], which a load fetches as
-// eight whole cache lines. Measured with these loads on all CUs and four
-// workgroups per XCD sharing a tile: 40 us per 2 MiB tile from 1 KiB runs, 50 us
-// from 64-byte row segments 4096 bytes apart (all hits: 20 against 35 us). The
-// block keeps that order in LDS; the fragment reads below allow for it.
-struct TileRows {
-  const unsigned char* wbase[LQ];  // uniform: where this wave's weight load q starts at k-step 0
-  const unsigned char* tbase;      // uniform: tokens, or this tile's h rows
-  unsigned wkstride;               // uniform: bytes from one k-step's weights to the next
-  unsigned tkstride;               // uniform: the same for the token rows
-  bool wpacked;                    // uniform: weight blocks are 1 KiB runs
-  bool tpacked;                    // uniform: so are the token blocks (the down projection's h rows)
-  unsigned woff[LQ];               // byte offset of this lane's 16 bytes of weight load q
-  unsigned toff[LQ];               // token stage: this lane's chunk of stage row wave*16*LQ+q*16+(lane>>2)
-};
-static_assert(G1_NB == 2 && G2_NB == 4, "the tiled variant reads the packed copy as 32+32-row and 64-row tasks");
-
-
-struct Frags {
-  uint4 a[4];   // weight blocks
-  uint4 b[WJ];  // token blocks
-};
-
-// Interleave hint for one half k-step: the 4 + WJ LDS reads spread evenly
-// between the 4 * WJ matrix instructions.
-__device__ __forceinline__ void interleave_reads_and_mfma() {
-  constexpr int PER = (4 * WJ) / (4 + WJ);
-#pragma unroll
-  for (int n = 0; n < 4 + WJ; ++n) {
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // DS read
-    __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // MFMA
-  }
-}
-
-// acc[i][j] (+)= W-block i (32 weight rows) x token-block j (32 token rows).
-// wblk[i]: first weight row of block i inside the weight stage; tokens of this
-// wave start at tok0. JMAX: token blocks of this wave that are computed.
-// Every wave loads its share of the weight rows of each stage whatever its
-// JMAX; TOKL: it also loads its 32 token rows (false when they all lie past the
-// tile's end: those stage rows then keep whatever they held, and feed only
-// output rows that the epilogue drops).
-template <int JMAX, bool TOKL>
-__device__ __forceinline__ void tile_gemm_j(const TileRows& rows, int ksteps, const int (&wblk)[4],
-                                            int tok0, f32x16 (&acc)[4][WJ]) {
-  constexpr int NLQ = TOKL ? 2 * LQ : LQ;  // this wave's loads per stage
-  const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
-  const int r32 = lane & 31, kq = lane >> 5;
-  const unsigned char* lds = lds_raw;
-  const unsigned lds_addr = uni(static_cast<unsigned>(
-      reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
-
-  // load q (0..LQ-1: weight rows, LQ..2*LQ-1: token rows) of this wave's loads
-  // of k-step ks into stage ks % STAGES
-  auto issue_one = [&](int ks, int q) {
-    const int src = ks;
-    const unsigned st = lds_addr + (ks & (STAGES - 1)) * STAGE_BYTES + wave * (LQ * 1024);
-    if (q < LQ) {
-      load_to_lds(rows.woff[q], rows.wbase[q] + static_cast<size_t>(src) * rows.wkstride, st + q * 1024);
+// One wave per SIMD, each with 64 weight rows x all token rows of the tile:
+// acc[2][JT] blocks of 32x32. The first 8 token blocks' accumulators fill the
+// 256 accumulator registers a[0:255]; a tile of 257..320 rows (JT 9, 10) keeps
+// the last blocks' in v[...]. Per 16 k a wave reads 2 weight and JT token
+// fragments (16 bytes per lane each) for 2*JT matrix instructions. A tile's
+// time follows its rows down to about 160; below that the 32 load round trips
+// of its k-loop set it.
+//
+// LDS stage layout: rows of 128 bytes, unpadded, weight rows 0..255 then token
+// rows. Row R keeps its eight 16-byte chunks permuted: chunk C sits at position
+// C ^ ((R >> 1) & 7), so the 16 rows a quarter-wave reads together at one k fall
+// into 16 different 16-byte bank groups. One wave-wide load fills 8 rows; lane
+// l brings the chunk that belongs at position l & 7 of row l >> 3.
+//
+// The matrix instructions are written as assembly with the accumulator pinned
+// to its register file: 256 accumulators fill a[0:255] exactly, and the
+// compiler's own choice moved parts of them in and out of v[...] (it also
+// chose the vector-register form of the instruction, which cannot reach a[...]).
+// The first instruction of every accumulator takes the constant 0 as its
+// addend, so nothing zeroes them.
+template <bool INIT, bool IN_V>
+__device__ __forceinline__ void mma32(const uint4& a, const uint4& b, f32x16& c) {
+  typedef unsigned v4u __attribute__((ext_vector_type(4)));
+  const v4u av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
+  if (IN_V) {
+    if (INIT) {
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(av), "v"(bv));
     } else {
-      load_to_lds(rows.toff[q - LQ], rows.tbase + static_cast<size_t>(src) * rows.tkstride,
-                  st + TN * TK * 2 + (q - LQ) * 1024);
-    }
-  };
-  auto issue = [&](int ks) {
-#pragma unroll
-    for (int q = 0; q < NLQ; ++q) issue_one(ks, q);
-  };
-
-  // per-lane read offsets: row r32 of a block, chunk kk*2+kq at its permuted position
-  const int swz = (r32 >> 2) & 3;
-  const int rd0 = r32 * 64 + ((kq ^ swz) << 4);        // kk = 0
-  const int rd1 = r32 * 64 + (((kq ^ swz) ^ 2) << 4);  // kk = 1
-
-  // packed weight blocks: row r32 of a 32-row block is row r32 % 16 of its 16-row
-  // block r32 / 16, chunk C of it at ((C * 16) + row) * 16
-  const int ra0 = rows.wpacked ? (r32 >> 4) * 1024 + ((kq * 16 + (r32 & 15)) << 4) : rd0;
-  const int ra1 = rows.wpacked ? (r32 >> 4) * 1024 + (((2 + kq) * 16 + (r32 & 15)) << 4) : rd1;
-  auto read_a = [&](Frags& f, int ks, int kk, int i) {
-    const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? ra0 : ra1);
-    if (JMAX > 0) f.a[i] = *reinterpret_cast<const uint4*>(st + wblk[i] * 64);
-  };
-  const int pk0 = (r32 >> 4) * 1024 + ((kq * 16 + (r32 & 15)) << 4);
-  const int pk1 = (r32 >> 4) * 1024 + (((2 + kq) * 16 + (r32 & 15)) << 4);
-  const int rb0 = rows.tpacked ? pk0 : rd0;
-  const int rb1 = rows.tpacked ? pk1 : rd1;
-  auto read_b = [&](Frags& f, int ks, int kk, int j) {
-    const unsigned char* st = lds + (ks & (STAGES - 1)) * STAGE_BYTES + (kk == 0 ? rb0 : rb1);
-    if (j < JMAX) f.b[j] = *reinterpret_cast<const uint4*>(st + TN * TK * 2 + (tok0 + j * 32) * 64);
-  };
-  auto read = [&](Frags& f, int ks, int kk) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) read_a(f, ks, kk, i);
-#pragma unroll
-    for (int j = 0; j < WJ; ++j) read_b(f, ks, kk, j);
-  };
-  auto mfma_block = [&](const Frags& f, int j) {
-    if (j < JMAX) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc[i][j] = mma32(f.a[i], f.b[j], acc[i][j]);
-      }
-    }
-  };
-
-  // k-step ks: fragments of its first half are in f0 on entry. While the first
-  // half multiplies, the second half is read; while the second half multiplies,
-  // the next stage is confirmed, the stage just finished is refilled, and the
-  // next step's first half is read — loads and reads spread between the matrix
-  // instructions. PENDING: loads of later stages that may still be in flight
-  // when stage ks+1 has to be complete (2 * LQ per stage).
-  Frags f0, f1;
-  auto step = [&](int ks, auto pending_tag, auto refill_tag, auto last_tag) {
-    constexpr int PENDING = decltype(pending_tag)::value;
-    constexpr int REFILL = decltype(refill_tag)::value;  // 1: refill with stage ks+STAGES
-    constexpr bool LAST = decltype(last_tag)::value;
-    read(f1, ks, 1);
-#pragma unroll
-    for (int j = 0; j < WJ; ++j) mfma_block(f0, j);
-    interleave_reads_and_mfma();
-    __builtin_amdgcn_sched_barrier(0);
-    if (!LAST) {
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // nobody still reads stage ks after the barrier
-      wait_vm<PENDING>();
-      __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
-#pragma unroll
-      for (int g = 0; g < WJ; ++g) {
-        mfma_block(f1, g);
-        __builtin_amdgcn_sched_barrier(0);
-        if (REFILL == 1) {
-          if (2 * g < NLQ) issue_one(ks + STAGES, 2 * g);
-          if (2 * g + 1 < NLQ) issue_one(ks + STAGES, 2 * g + 1);
-        }
-
-#pragma unroll
-        for (int i = g * (4 / WJ); i < (g + 1) * (4 / WJ); ++i) read_a(f0, ks + 1, 0, i);
-        read_b(f0, ks + 1, 0, g);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < WJ; ++j) mfma_block(f1, j);
-    }
-  };
-  using I0 = std::integral_constant<int, 0>;
-  using I8 = std::integral_constant<int, NLQ>;       // one later stage in flight
-  using I16 = std::integral_constant<int, 2 * NLQ>;  // two later stages in flight
-
-  using R0 = std::integral_constant<int, 0>;
-  using R1 = std::integral_constant<int, 1>;
-#pragma unroll
-  for (int s = 0; s < STAGES; ++s) issue(s);  // ksteps >= STAGES for every admitted shape
-  wait_vm<3 * NLQ>();
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-  read(f0, 0, 0);
-  int ks = 0;
-  for (; ks + STAGES < ksteps; ++ks) step(ks, I16{}, R1{}, std::false_type{});
-  step(ks++, I16{}, R0{}, std::false_type{});
-  step(ks++, I8{}, R0{}, std::false_type{});
-  step(ks++, I0{}, R0{}, std::false_type{});
-  step(ks, I0{}, R0{}, std::true_type{});
-  __syncthreads();  // the stages are free for the epilogue
-}
-
-// jmax is the same for the whole wave: one straight-line loop body per value.
-// Rounding it up is safe: rows past the tile's end are clamped copies whose
-// results the epilogue drops.
-__device__ __forceinline__ void tile_gemm(const TileRows& rows, int ksteps, const int (&wblk)[4],
-                                          int tok0, int jmax, bool tokl, f32x16 (&acc)[4][WJ]) {
-  if (tokl) {
-    if (jmax > WJ / 2) {
-      tile_gemm_j<WJ, true>(rows, ksteps, wblk, tok0, acc);
-    } else if (jmax > 0) {
-      tile_gemm_j<WJ / 2, true>(rows, ksteps, wblk, tok0, acc);
-    } else {
-      tile_gemm_j<0, true>(rows, ksteps, wblk, tok0, acc);
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
     }
   } else {
-    if (jmax > WJ / 2) {
-      tile_gemm_j<WJ, false>(rows, ksteps, wblk, tok0, acc);
-    } else if (jmax > 0) {
-      tile_gemm_j<WJ / 2, false>(rows, ksteps, wblk, tok0, acc);
+    if (INIT) {
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(av), "v"(bv));
     } else {
-      tile_gemm_j<0, false>(rows, ksteps, wblk, tok0, acc);
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
     }
   }
 }
 
-// The chunk lane `lane` of wave `wave` loads for stage row wave*16*LQ + q*16 + (lane >> 2):
-// position lane & 3 of that row holds chunk (lane & 3) ^ ((row >> 2) & 3).
-__device__ __forceinline__ int stage_row(int q) {
-  return (threadIdx.x >> 6) * (16 * LQ) + q * 16 + ((threadIdx.x & 63) >> 2);
+constexpr int ntl_of(int jt) { return jt > 8 ? 10 : 8; }            // 8-row token loads per wave and stage
+constexpr int stage_bytes_of(int jt) { return (TN + 4 * 8 * ntl_of(jt)) * ROWB; }
+constexpr int TILE_LDS_BYTES = 2 * stage_bytes_of(JT_MAX);          // 147456
+// behind the stages: the tile's destination rows and gate weights for the down epilogue
+constexpr int SIDE_OFF = TILE_LDS_BYTES;
+constexpr int SIDE_BYTES = TM_MAX * 8;
+// and behind those one 16-byte line of words a GEMM task leaves for the worker loop: the ticket it
+// drew for the workgroup's next task, and (timing experiments) its phase times. They live in
+// the dynamic block because a file-scope LDS variable written from a function that is not
+// inlined landed on top of the dynamic block's first bytes.
+constexpr int NOTE_OFF = SIDE_OFF + SIDE_BYTES;
+constexpr int NOTE_BYTES = 16;
+__device__ __forceinline__ unsigned* task_notes() { return reinterpret_cast<unsigned*>(lds_raw + NOTE_OFF); }
+constexpr int EPI_LD = TN * 2 + 16;              // bytes per row of the down epilogue's staging slab
+static_assert(128 * EPI_LD <= TILE_LDS_BYTES, "epilogue slab exceeds the stage buffers");
+
+struct TileOperands {
+  const unsigned char* wbase;  // uniform: the weight matrix the offsets are relative to
+  const unsigned char* tbase;  // uniform: tokens, or h
+  unsigned woff[NLD];          // this lane's 16 bytes of weight load q at stage 0
+  unsigned toff[10];           // the same for the token rows
+};
+
+// Stage row (within its operand) that this lane's part of load q belongs to when a wave
+// issues `per_wave` loads per stage, and the byte offset inside the row's 128-byte line of
+// the chunk it brings.
+__device__ __forceinline__ int stage_row(int per_wave, int q) {
+  return ((threadIdx.x >> 6) * per_wave + q) * 8 + ((threadIdx.x & 63) >> 3);
 }
 __device__ __forceinline__ unsigned stage_chunk_bytes(int row) {
-  return static_cast<unsigned>(((threadIdx.x & 3) ^ ((row >> 2) & 3)) << 4);
+  return static_cast<unsigned>(((threadIdx.x & 7) ^ ((row >> 1) & 7)) << 4);
 }
 
-// h of the tiled variant: row tile m owns HT_ROWS rows x I, stored the way the down
-// projection's loads want them: [k-step of 32 columns][16-row block][chunk 0..3][row 0..15][16 B],
-// so a block of a k-step is one 1 KiB run.
-__device__ __forceinline__ size_t tiled_h_tile_bytes(int I) { return static_cast<size_t>(HT_ROWS) * I * 2; }
-
-// gate/up: h[row, n0 .. n0+128) for one row tile
-// (test/singleGPU/cpp/moe/reference/refExpertFFN1.h:51-65).
-__device__ __noinline__ void tiled_gateup_task(ParamsRef pv, const TileDesc& tile_in, int m, int nblk) {
-  ParamsRef p = uniform_params(pv);
-  const int H = uni(p.H), I = uni(p.I), K = uni(p.K);
-  TileDesc tile;
-  tile.expert = uni(tile_in.expert);
-  tile.row0 = uni(tile_in.row0);
-  tile.rows = uni(tile_in.rows);
-  const int n0 = uni(nblk) * G1_COLS;
-  const unsigned short* w13 = uni(reinterpret_cast<const unsigned short*>(p.ffn1)) +
-                              static_cast<size_t>(tile.expert) * 2 * I * H;
-  TileRows rows;
-  rows.wpacked = uni(p.ffn1_packed != nullptr ? 1 : 0) != 0;
-  rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
-  rows.tkstride = static_cast<unsigned>(TK * 2);
-  rows.tpacked = false;
-  rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
-#pragma unroll
-  for (int q = 0; q < LQ; ++q) {
-    const int row = stage_row(q);
-    if (rows.wpacked) {
-      // stage block B (16 rows): gate blocks 0..7, up blocks 8..15; the packed task
-      // of 32 h columns holds gate blocks 0,1 and up blocks 2,3 of every k-step
-      const int B = uni(static_cast<int>(threadIdx.x >> 6)) * LQ + q;
-      const int half = B >> 3, b8 = B & 7;
-      const size_t task = static_cast<size_t>(tile.expert) * (I / 32) + (n0 / 32 + (b8 >> 1));
-      rows.wbase[q] = uni(reinterpret_cast<const unsigned char*>(p.ffn1_packed)) +
-                      task * (static_cast<size_t>(H / 32) * 4096) + (2 * half + (b8 & 1)) * 1024;
-      rows.woff[q] = (threadIdx.x & 63) * 16;
-    } else {
-      // weight stage rows 0..127: gate rows n0+row, 128..255: up rows I+n0+(row-128)
-      const int wrow = row < G1_COLS ? n0 + row : I + n0 + (row - G1_COLS);
-      rows.wbase[q] = reinterpret_cast<const unsigned char*>(w13);
-      rows.woff[q] = static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
-    }
-    const int tok = ldc(&p.perm[tile.row0 + min(row, tile.rows - 1)]) / K;
-    rows.toff[q] = static_cast<unsigned>(tok) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
-  }
-  const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int wn = wave & 1, wm = wave >> 1;
-  const int wblk[4] = {wn * 64, wn * 64 + 32, G1_COLS + wn * 64, G1_COLS + wn * 64 + 32};
-  const int tok0 = wm * (32 * WJ);
-  const int jmax = uni(min(WJ, max(0, (tile.rows - tok0 + 31) / 32)));
-  const bool tokl = wave * (16 * LQ) < tile.rows;  // some of the token rows this wave loads exist
-  // this wave's 64 columns are k-steps (n0 + 64*wn)/32 and the next of the tile's h
-  unsigned char* h = uni(reinterpret_cast<unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I) +
-                     static_cast<size_t>((n0 + wn * 64) / 32) * (HT_ROWS * 64);
-  f32x16 acc[4][WJ];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < WJ; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-  tile_gemm(rows, H / TK, wblk, tok0, jmax, tokl, acc);
-
-  // Epilogue through LDS (the stage buffers are free now): each wave turns its
-  // 32-token x 64-column blocks into full 128-byte row segments of h. Nothing
-  // here waits for a store.
-  const int r32 = lane & 31, kq = lane >> 5;
-  constexpr int SLD = 64 + 8;  // slab row stride, bf16 elements
-  unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * 32 * SLD;
-#pragma unroll
-  for (int j = 0; j < WJ; ++j) {
-    if (j < jmax) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          float hv[4];
-#pragma unroll
-          for (int v = 0; v < 4; ++v)
-            hv[v] = silu_mul_fast(acc[i][j][g4 * 4 + v], acc[i + 2][j][g4 * 4 + v]);
-          uint2 pk;
-          pk.x = pack_bf16(hv[0], hv[1]);
-          pk.y = pack_bf16(hv[2], hv[3]);
-          *reinterpret_cast<uint2*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) = pk;
-        }
-      lds_wave_sync();
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        // one 1 KiB run: k-step it / 2 of this wave's two, 16-row block it % 2 of this token block
-        const int ksl = it >> 1, b16 = it & 1;
-        const int rr = b16 * 16 + (lane & 15), cc = ksl * 32 + (lane >> 4) * 8;
-        const int trow = tok0 + j * 32 + rr;
-        const uint4 v = *reinterpret_cast<const uint4*>(slab + rr * SLD + cc);
-        if (trow < tile.rows)
-          st16_through(h + static_cast<size_t>(ksl) * (HT_ROWS * 64) + ((tok0 + j * 32) / 16 + b16) * 1024 + lane * 16, v);
-      }
-      lds_wave_sync();
-    }
-  }
-}
-
-// down: y[t*K+slot, n0 .. n0+256) = w * (h[row] . W2[e]^T)
-// (refFullMoe.h:58-65, src/hip/kernel/tasks/ffn2Task.h:37-40).
-__device__ __noinline__ void tiled_down_task(ParamsRef pv, const TileDesc& tile_in, int m, int nblk) {
-  ParamsRef p = uniform_params(pv);
-  const int H = uni(p.H), I = uni(p.I);
-  TileDesc tile;
-  tile.expert = uni(tile_in.expert);
-  tile.row0 = uni(tile_in.row0);
-  tile.rows = uni(tile_in.rows);
-  const int n0 = uni(nblk) * TN;
-  const unsigned short* w2 = uni(reinterpret_cast<const unsigned short*>(p.ffn2)) +
-                             static_cast<size_t>(tile.expert) * H * I;
-  TileRows rows;
-  rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I);
-  rows.tkstride = static_cast<unsigned>(HT_ROWS * 64);
-  rows.tpacked = true;
-  rows.wpacked = uni(p.ffn2_packed != nullptr ? 1 : 0) != 0;
-  rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
-#pragma unroll
-  for (int q = 0; q < LQ; ++q) {
-    const int row = stage_row(q);
-    if (rows.wpacked) {
-      // stage block B (16 rows of W2): the packed task of 64 output columns holds its blocks 0..3
-      const int B = uni(static_cast<int>(threadIdx.x >> 6)) * LQ + q;
-      const size_t task = static_cast<size_t>(tile.expert) * (H / 64) + (n0 / 64 + (B >> 2));
-      rows.wbase[q] = uni(reinterpret_cast<const unsigned char*>(p.ffn2_packed)) +
-                      task * (static_cast<size_t>(I / 32) * 4096) + (B & 3) * 1024;
-      rows.woff[q] = (threadIdx.x & 63) * 16;
-    } else {
-      rows.wbase[q] = reinterpret_cast<const unsigned char*>(w2);
-      rows.woff[q] = static_cast<unsigned>(n0 + row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
-    }
-    // token stage block wave*LQ + q is one run of the tile's h (rows past the tile's
-    // end were never written; their products are dropped)
-    rows.toff[q] = static_cast<unsigned>((uni(static_cast<int>(threadIdx.x >> 6)) * LQ + q) * 1024 + (threadIdx.x & 63) * 16);
-  }
-  const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int wn = wave & 1, wm = wave >> 1;
-  const int wblk[4] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
-  const int tok0 = wm * (32 * WJ);
-  const int jmax = uni(min(WJ, max(0, (tile.rows - tok0 + 31) / 32)));
-  const bool tokl = wave * (16 * LQ) < tile.rows;  // some of the token rows this wave loads exist
-  const int r32 = lane & 31, kq = lane >> 5;
-  // y rows are bf16 here: H values per (token, slot)
-  unsigned short* y = uni(reinterpret_cast<unsigned short*>(p.y)) + n0 + wn * 128 + (lane & 15) * 8;
-  // gate weight and destination row (token*K + slot) of this lane's row in each token block
-  float roww[WJ];
-  int dstrow[WJ];
-  {
-    const float* row_w = uni(p.row_w) + tile.row0;
-    const int* perm = uni(p.perm) + tile.row0;
-#pragma unroll
-    for (int j = 0; j < WJ; ++j) {
-      const int myrow = tok0 + j * 32 + r32;
-      const bool valid = myrow < tile.rows;
-      roww[j] = valid ? ldc(&row_w[myrow]) : 0.0f;
-      dstrow[j] = valid ? ldc(&perm[myrow]) : -1;
-    }
-  }
-  f32x16 acc[4][WJ];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < WJ; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-  tile_gemm(rows, I / TK, wblk, tok0, jmax, tokl, acc);
-
-  // Epilogue through LDS: 32-token x 128-column blocks become 256-byte row
-  // segments of y (bf16), scaled by the row's gate weight, at the row's
-  // (token, slot). Nothing here waits for a store.
-  constexpr int SLD = 128 + 8;  // slab row stride, bf16 elements
-  unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * (32 * SLD);
-#pragma unroll
-  for (int j = 0; j < WJ; ++j) {
-    if (j < jmax) {
-      const float w = roww[j];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          uint2 pk;
-          pk.x = pack_bf16(acc[i][j][g4 * 4 + 0] * w, acc[i][j][g4 * 4 + 1] * w);
-          pk.y = pack_bf16(acc[i][j][g4 * 4 + 2] * w, acc[i][j][g4 * 4 + 3] * w);
-          *reinterpret_cast<uint2*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) = pk;
-        }
-      lds_wave_sync();
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        // each quarter-wave stores one row: rows 4*it .. 4*it+3
-        const int q = lane >> 4;
-        const int d0 = __builtin_amdgcn_readlane(dstrow[j], it * 4);
-        const int d1 = __builtin_amdgcn_readlane(dstrow[j], it * 4 + 1);
-        const int d2 = __builtin_amdgcn_readlane(dstrow[j], it * 4 + 2);
-        const int d3 = __builtin_amdgcn_readlane(dstrow[j], it * 4 + 3);
-        const int dst = q == 0 ? d0 : q == 1 ? d1 : q == 2 ? d2 : d3;
-        const uint4 v = *reinterpret_cast<const uint4*>(slab + (it * 4 + q) * SLD + (lane & 15) * 8);
-        if (dst >= 0) st16_through(y + static_cast<size_t>(dst) * H, v);
-      }
-      lds_wave_sync();
-    }
-  }
-}
-
-// ------------------------------------------------------------ tall row tiles
-// A row tile of 257..320 rows (an expert's last full tile plus its short tail):
-// one pass over the expert's weights instead of two. Waves are laid out 4 (64
-// weight rows, two blocks) x 2 (160 token rows, five blocks): 160 accumulator
-// registers per lane. A stage holds 256 weight rows and 320 token rows (36 KiB);
-// every wave loads two weight blocks, and token blocks wave, wave + 8 and (waves
-// 0..3) wave + 16 of the twenty 16-row blocks. Otherwise as tile_gemm_j.
-struct TallRows {
-  const unsigned char* wbase[LQ];
-  const unsigned char* tbase;
-  unsigned wkstride, tkstride;
-  bool wpacked, tpacked;
-  unsigned woff[LQ];
-  unsigned toff[3];
-};
-struct TallFrags {
-  uint4 a[2];  // weight blocks
-  uint4 b[5];  // token blocks
+struct Frag {
+  uint4 a[2];
+  uint4 b[JT_MAX];
 };
 
-// NTB: token blocks of this wave that are computed (4 or 5); NTL: its token loads per stage (2 or 3)
-template <int NTB, int NTL>
-__device__ __forceinline__ void tall_gemm(const TallRows& rows, int ksteps, const int (&wblk)[2], int tok0,
-                                          f32x16 (&acc)[2][5]) {
-  constexpr int NLD = LQ + NTL;  // this wave's loads per stage
-  static_assert(LQ == 2 && NLD <= 5, "tall tiles are written for eight waves");
+// acc[i][j] = W-block i (32 of this wave's 64 weight rows) x token-block j, j < JT, over
+// nstages * 64 k (nstages >= 2). Token rows from 32*JT on are neither loaded nor multiplied.
+//
+// A stage is 4 sub-steps of 16 k; a sub-step is NS = max(8, JT) slots; a slot is one pair of
+// matrix instructions and, behind it, the LDS reads and global loads the schedule puts there:
+//  * the fragments of sub-step u+1 are read under sub-step u, one token block per slot
+//  * hand-over in sub-step 3 after BAR pairs: this wave's reads of stage s have returned and
+//    its loads of stage s+1 have landed, then the workgroup barrier; from there on the next
+//    stage's first fragments are read and the loads of stage s+2 go out into the buffer just
+//    left, one per slot, the rest under the next stage's first sub-steps. (Measured on all
+//    256 CUs: all 16 loads behind the barrier at once, barrier in front of the sub-step: 51 us
+//    per 256x256x2048 tile; this schedule: 48 us.)
+//
+// Bookkeeping rides along: at the first hand-over (every memory operation this wave issued
+// before it, the previous task's stores included, has completed there anyway) thread 0
+// signals the previous task's completion on `pend` (if any) and draws the workgroup's next
+// ticket from `queue` into `next`, so neither trip to memory is waited for between tasks.
+template <int JT>
+__device__ __forceinline__ void tile_gemm(const TileOperands& op, int nstages, f32x16 (&acc)[2][JT_MAX],
+                                          unsigned* pend, unsigned* queue, unsigned& next) {
   const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
   const int r32 = lane & 31, kq = lane >> 5;
-  const unsigned char* lds = lds_raw;
   const unsigned lds_addr = uni(static_cast<unsigned>(
       reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
+  constexpr int TROWS = 32 * JT;
+  constexpr int NTL = ntl_of(JT);
+  constexpr int STG = stage_bytes_of(JT);
+  constexpr int NS = JT > 8 ? JT : 8;  // slots per sub-step
+  constexpr int NRD = 2 + JT;          // fragment reads per sub-step
+  constexpr int BAR = 2;               // pairs of sub-step 3 in front of the hand-over
+  constexpr int AFTER = NS - BAR;      // slots of sub-step 3 behind it
+  constexpr int RPS = (NRD + AFTER - 1) / AFTER;  // reads of the next stage's first fragments per slot there
 
-  auto issue_one = [&](int ks, int q) {
-    const unsigned st = lds_addr + (ks & (STAGES - 1)) * TALL_STAGE_BYTES;
-    if (q < LQ) {
-      load_to_lds(rows.woff[q], rows.wbase[q] + static_cast<size_t>(ks) * rows.wkstride,
-                  st + (wave * LQ + q) * 1024);
-    } else {
-      load_to_lds(rows.toff[q - LQ], rows.tbase + static_cast<size_t>(ks) * rows.tkstride,
-                  st + TN * TK * 2 + (wave + 8 * (q - LQ)) * 1024);
+  int fo[4];  // per-lane fragment offsets of the four 16-k sub-steps
+#pragma unroll
+  for (int u = 0; u < 4; ++u) fo[u] = r32 * ROWB + (((2 * u + kq) ^ ((r32 >> 1) & 7)) << 4);
+
+  auto issue_one = [&](int s, int q) {  // q: 0..7 weights, 8..8+NTL-1 tokens
+    const unsigned st = uni(static_cast<int>(lds_addr + (s & 1) * STG));
+    if (q < NLD) {
+      load_to_lds(op.woff[q], op.wbase + static_cast<size_t>(s) * ROWB, st + (wave * 64 + q * 8) * ROWB);
+    } else if (q < NLD + NTL) {
+      const int qq = q - NLD;
+      if ((NTL == 8 && JT == 8) || (wave * NTL + qq) * 8 < TROWS)
+        load_to_lds(op.toff[qq], op.tbase + static_cast<size_t>(s) * ROWB,
+                    st + TN * ROWB + ((wave * NTL + qq) * 8) * ROWB);
     }
   };
-  auto issue = [&](int ks) {
-#pragma unroll
-    for (int q = 0; q < NLD; ++q) issue_one(ks, q);
-  };
-
-  const int swz = (r32 >> 2) & 3;
-  const int rd0 = r32 * 64 + ((kq ^ swz) << 4);
-  const int rd1 = r32 * 64 + (((kq ^ swz) ^ 2) << 4);
-  const int pk0 = (r32 >> 4) * 1024 + ((kq * 16 + (r32 & 15)) << 4);
-  const int pk1 = (r32 >> 4) * 1024 + (((2 + kq) * 16 + (r32 & 15)) << 4);
-  const int ra0 = rows.wpacked ? pk0 : rd0, ra1 = rows.wpacked ? pk1 : rd1;
-  const int rb0 = rows.tpacked ? pk0 : rd0, rb1 = rows.tpacked ? pk1 : rd1;
-  auto read_a = [&](TallFrags& f, int ks, int kk, int i) {
-    const unsigned char* st = lds + (ks & (STAGES - 1)) * TALL_STAGE_BYTES + (kk == 0 ? ra0 : ra1);
-    f.a[i] = *reinterpret_cast<const uint4*>(st + wblk[i] * 64);
-  };
-  auto read_b = [&](TallFrags& f, int ks, int kk, int j) {
-    const unsigned char* st = lds + (ks & (STAGES - 1)) * TALL_STAGE_BYTES + (kk == 0 ? rb0 : rb1);
-    if (j < NTB) f.b[j] = *reinterpret_cast<const uint4*>(st + TN * TK * 2 + (tok0 + j * 32) * 64);
-  };
-  auto read = [&](TallFrags& f, int ks, int kk) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) read_a(f, ks, kk, i);
-#pragma unroll
-    for (int j = 0; j < 5; ++j) read_b(f, ks, kk, j);
-  };
-  auto mfma_block = [&](const TallFrags& f, int j) {
-    if (j < NTB) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i) acc[i][j] = mma32(f.a[i], f.b[j], acc[i][j]);
+  auto read_n = [&](Frag& f, int s, int u, int r) {  // r-th of the NRD reads of a sub-step
+    const unsigned char* st = lds_raw + (s & 1) * STG + fo[u];
+    if (r < 2) {
+      f.a[r] = *reinterpret_cast<const uint4*>(st + (wave * 64 + r * 32) * ROWB);
+    } else if (r < NRD) {
+      f.b[r - 2] = *reinterpret_cast<const uint4*>(st + TN * ROWB + ((r - 2) * 32) * ROWB);
     }
   };
-
-  TallFrags f0, f1;
-  auto step = [&](int ks, auto pending_tag, auto refill_tag, auto last_tag) {
-    constexpr int PENDING = decltype(pending_tag)::value;
-    constexpr int REFILL = decltype(refill_tag)::value;
-    constexpr bool LAST = decltype(last_tag)::value;
-    read(f1, ks, 1);
-#pragma unroll
-    for (int j = 0; j < 5; ++j) mfma_block(f0, j);
-#pragma unroll
-    for (int n = 0; n < 2 + NTB; ++n) {  // the reads spread between the matrix instructions
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+  auto pair = [&](auto init_tag, const Frag& cur, int j) {
+    constexpr bool INIT = decltype(init_tag)::value;
+    if (j < JT) {
+      if (j < 8) {
+        mma32<INIT, false>(cur.a[0], cur.b[j], acc[0][j]);
+        mma32<INIT, false>(cur.a[1], cur.b[j], acc[1][j]);
+      } else {
+        mma32<INIT, true>(cur.a[0], cur.b[j], acc[0][j]);
+        mma32<INIT, true>(cur.a[1], cur.b[j], acc[1][j]);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (!LAST) {
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // nobody still reads stage ks after the barrier
-      wait_vm<PENDING>();
-      __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
-#pragma unroll
-      for (int g = 0; g < 5; ++g) {
-        mfma_block(f1, g);
-        __builtin_amdgcn_sched_barrier(0);
-        if (REFILL == 1 && g < NLD) issue_one(ks + STAGES, g);
-        if (g < 2) read_a(f0, ks + 1, 0, g);
-        read_b(f0, ks + 1, 0, g);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 5; ++j) mfma_block(f1, j);
+  };
+
+  auto bookkeeping = [&]() {
+    if (threadIdx.x == 0) {
+      if (pend != nullptr) (void)add_relaxed(pend, 1u);
+      next = add_relaxed(queue, 1u);
     }
   };
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, NLD>;
-  using I2 = std::integral_constant<int, 2 * NLD>;
-  using R0 = std::integral_constant<int, 0>;
-  using R1 = std::integral_constant<int, 1>;
+
+  Frag f0, f1;
 #pragma unroll
-  for (int st = 0; st < STAGES; ++st) issue(st);
-  wait_vm<3 * NLD>();
+  for (int q = 0; q < NLD + NTL; ++q) issue_one(0, q);
+#pragma unroll
+  for (int q = 0; q < NLD + NTL; ++q) issue_one(1, q);
+  // stage 0 has landed (this wave's part; stage 1 may be in flight), then everybody's
+  {
+    // live token loads of this wave per stage
+    const int ntl = uni(max(0, min(NTL, (TROWS - wave * NTL * 8 + 7) / 8)));
+    const int keep = 8 + ntl;  // loads of stage 1 that may stay in flight
+    if (keep >= 18) {
+      wait_vm<18>();
+    } else if (keep >= 16) {
+      wait_vm<16>();
+    } else if (keep >= 12) {
+      wait_vm<12>();
+    } else {
+      wait_vm<8>();
+    }
+  }
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  read(f0, 0, 0);
-  int ks = 0;
-  for (; ks + STAGES < ksteps; ++ks) step(ks, I2{}, R1{}, std::false_type{});
-  step(ks++, I2{}, R0{}, std::false_type{});
-  step(ks++, I1{}, R0{}, std::false_type{});
-  step(ks++, I0{}, R0{}, std::false_type{});
-  step(ks, I0{}, R0{}, std::true_type{});
+#pragma unroll
+  for (int r = 0; r < NRD; ++r) read_n(f0, 0, 0, r);
+
+  auto stage = [&](int s, auto first_tag, auto early_tag, auto late_tag, auto next_tag) {
+    constexpr bool EARLY = decltype(early_tag)::value;  // the tail of stage s+1's loads is still to go out
+    constexpr bool LATE = decltype(late_tag)::value;    // stage s+2 exists
+    constexpr bool NEXT = decltype(next_tag)::value;    // stage s+1 exists
+    using No = std::false_type;
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      const Frag& cur = (u & 1) ? f1 : f0;
+      Frag& nxt = (u & 1) ? f0 : f1;
+#pragma unroll
+      for (int j = 0; j < NS; ++j) {
+        if (u == 0) {
+          pair(first_tag, cur, j);
+        } else {
+          pair(No{}, cur, j);
+        }
+        if (EARLY) issue_one(s + 1, AFTER + NS * u + j);
+        if (j == 0) {
+          read_n(nxt, s, u + 1, 0);
+          read_n(nxt, s, u + 1, 1);
+        }
+        read_n(nxt, s, u + 1, 2 + j);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+      if (j == BAR) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (NEXT) {
+          wait_vm<0>();
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+          if (decltype(first_tag)::value) bookkeeping();
+        }
+      }
+      pair(No{}, f1, j);
+      if (j >= BAR) {
+        if (LATE) issue_one(s + 2, j - BAR);
+        if (NEXT) {
+#pragma unroll
+          for (int r = (j - BAR) * RPS; r < (j - BAR + 1) * RPS; ++r) read_n(f0, s + 1, 0, r);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+  if (nstages > 2) {
+    stage(0, Yes{}, No{}, Yes{}, Yes{});
+  } else {
+    stage(0, Yes{}, No{}, No{}, Yes{});
+  }
+  int s = 1;
+  for (; s + 2 < nstages; ++s) stage(s, No{}, Yes{}, Yes{}, Yes{});
+  if (s + 1 < nstages) {
+    stage(s, No{}, Yes{}, No{}, Yes{});
+    ++s;
+  }
+  stage(s, No{}, No{}, No{}, No{});
+  // the compiler does not see matrix instructions in the assembly above: keep the wait states
+  // between the last of them and the first read of an accumulator
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   __syncthreads();  // the stages are free for the epilogue
 }
 
-// dispatch on the wave's position: waves 0..3 own token rows 0..159 (all five blocks live, three
-// token loads), waves 4..7 rows 160..319 (four or five blocks, two loads)
-__device__ __forceinline__ void tall_gemm_dispatch(const TallRows& rows, int ksteps, const int (&wblk)[2],
-                                                   int tok0, int ntb, f32x16 (&acc)[2][5]) {
-  if (uni(static_cast<int>(threadIdx.x >> 6)) < 4) {
-    tall_gemm<5, 3>(rows, ksteps, wblk, tok0, acc);
-  } else if (ntb > 4) {
-    tall_gemm<5, 2>(rows, ksteps, wblk, tok0, acc);
-  } else {
-    tall_gemm<4, 2>(rows, ksteps, wblk, tok0, acc);
-  }
-}
-
-// the 16-row token block L (0..19) this wave loads as its q-th token load, or -1
-__device__ __forceinline__ int tall_token_block(int q) {
-  const int L = static_cast<int>(threadIdx.x >> 6) + 8 * q;
-  return L < TALL_TM / 16 ? L : -1;
-}
-
-__device__ __noinline__ void tall_gateup_task(ParamsRef pv, const TileDesc& tile_in, int m, int nblk) {
-  ParamsRef p = uniform_params(pv);
+// One GEMM tile task, gate/up or down, for a row tile of up to 32*JT rows.
+//
+// gate/up: h[row, n0 .. n0+128) (test/singleGPU/cpp/moe/reference/refExpertFFN1.h:51-65).
+// h is [T*K, I] row-major, rows in permuted order. Wave w holds gate rows n0+32w.. and the
+// matching up rows, so SiLU(gate)*up happens in registers; the tile's 128 columns leave
+// through LDS as 256-byte row segments.
+//
+// down: y[t*K+slot, n0 .. n0+256) = w * (h[row] . W2[e]^T) (refFullMoe.h:58-65,
+// src/hip/kernel/tasks/ffn2Task.h:37-40), bf16, through LDS as 512-byte row segments, 128
+// rows at a time. The rows' destinations and gate weights are fetched when the task starts
+// and parked in LDS behind the stages, so the epilogue waits for no memory.
+template <int JT, bool down>
+__device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int rows, int nblk, unsigned* pend,
+                                          unsigned* queue) {
+#ifdef FMOE_TRACE_PHASES
+  const long long ph0 = wall_clock64();
+#endif
   const int H = uni(p.H), I = uni(p.I), K = uni(p.K);
-  TileDesc tile;
-  tile.expert = uni(tile_in.expert);
-  tile.row0 = uni(tile_in.row0);
-  tile.rows = uni(tile_in.rows);
-  const int n0 = uni(nblk) * G1_COLS;
   const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const unsigned short* w13 = uni(reinterpret_cast<const unsigned short*>(p.ffn1)) +
-                              static_cast<size_t>(tile.expert) * 2 * I * H;
-  TallRows rows;
-  rows.wpacked = uni(p.ffn1_packed != nullptr ? 1 : 0) != 0;
-  rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
-  rows.tkstride = static_cast<unsigned>(TK * 2);
-  rows.tpacked = false;
-  rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
+  constexpr int NTL = ntl_of(JT);
+  const int* perm = uni(p.perm) + row0;
+  const int n0 = uni(nblk) * (down ? TN : G1_COLS);
+  TileOperands op;
+  int side_dst[2];
+  float side_w[2];
+  int nstages;
+  if (down) {
+    nstages = I / KS;
+    op.wbase = uni(reinterpret_cast<const unsigned char*>(p.ffn2)) + (static_cast<size_t>(expert) * H + n0) * I * 2;
+    op.tbase = uni(reinterpret_cast<const unsigned char*>(p.h)) + static_cast<size_t>(row0) * I * 2;
+    const float* row_w = uni(p.row_w) + row0;
 #pragma unroll
-  for (int q = 0; q < LQ; ++q) {
-    const int row = stage_row(q);
-    if (rows.wpacked) {
-      const int B = wave * LQ + q;
-      const int half = B >> 3, b8 = B & 7;
-      const size_t task = static_cast<size_t>(tile.expert) * (I / 32) + (n0 / 32 + (b8 >> 1));
-      rows.wbase[q] = uni(reinterpret_cast<const unsigned char*>(p.ffn1_packed)) +
-                      task * (static_cast<size_t>(H / 32) * 4096) + (2 * half + (b8 & 1)) * 1024;
-      rows.woff[q] = lane * 16;
-    } else {
-      const int wrow = row < G1_COLS ? n0 + row : I + n0 + (row - G1_COLS);
-      rows.wbase[q] = reinterpret_cast<const unsigned char*>(w13);
-      rows.woff[q] = static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+    for (int k = 0; k < 2; ++k) {
+      const int r = static_cast<int>(threadIdx.x) + k * T_THREADS;
+      side_dst[k] = r < rows ? ldc(&perm[r]) : -1;
+      side_w[k] = r < rows ? ldc(&row_w[r]) : 0.0f;
+    }
+#pragma unroll
+    for (int q = 0; q < NLD; ++q) {
+      const int row = stage_row(NLD, q);
+      op.woff[q] = static_cast<unsigned>(row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
+    }
+#pragma unroll
+    for (int q = 0; q < NTL; ++q) {
+      const int row = stage_row(NTL, q);
+      op.toff[q] = static_cast<unsigned>(min(row, rows - 1)) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
+    }
+  } else {
+    nstages = H / KS;
+    op.wbase = uni(reinterpret_cast<const unsigned char*>(p.ffn1)) + static_cast<size_t>(expert) * 2 * I * H * 2;
+    op.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
+#pragma unroll
+    for (int q = 0; q < NLD; ++q) {
+      const int row = stage_row(NLD, q);
+      // weight stage rows 64w..64w+31: gate rows n0+32w.., 64w+32..64w+63: up rows I+n0+32w..
+      const int wl = row & 63;
+      const int wrow = (wl < 32 ? n0 : I + n0 - 32) + 32 * wave + wl;
+      op.woff[q] = static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+    }
+#pragma unroll
+    for (int q = 0; q < NTL; ++q) {
+      const int row = stage_row(NTL, q);
+      const int tok = ldc(&perm[min(row, rows - 1)]) / K;
+      op.toff[q] = static_cast<unsigned>(tok) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
     }
   }
-#pragma unroll
-  for (int q = 0; q < 3; ++q) {
-    const int L = max(tall_token_block(q), 0);
-    const int row = L * 16 + (lane >> 2);
-    const int tok = ldc(&p.perm[tile.row0 + min(row, tile.rows - 1)]) / K;
-    rows.toff[q] = static_cast<unsigned>(tok) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+  f32x16 acc[2][JT_MAX];
+#ifdef FMOE_TRACE_PHASES
+  const long long ph1 = wall_clock64();
+  const long long pc1 = clock64();
+#endif
+  unsigned next = 0u;
+  tile_gemm<JT>(op, nstages, acc, pend, queue, next);
+  if (threadIdx.x == 0) task_notes()[0] = next;  // the epilogue's barriers publish it
+#ifdef FMOE_TRACE_PHASES
+  if (threadIdx.x == 0) {
+    task_notes()[1] = static_cast<unsigned>(ph1 - ph0);
+    task_notes()[2] = static_cast<unsigned>(wall_clock64() - ph1) | (static_cast<unsigned>((clock64() - pc1) >> 6) << 16);
   }
-  const int wn = wave & 3, wm = wave >> 2;
-  const int wblk[2] = {wn * 32, G1_COLS + wn * 32};  // 32 gate rows and the matching 32 up rows
-  const int tok0 = wm * 160;
-  const int ntb = uni(min(5, (tile.rows - tok0 + 31) / 32));
-  // this wave's 32 columns are k-step (n0 + 32*wn)/32 of the tile's h
-  unsigned char* h = uni(reinterpret_cast<unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I) +
-                     static_cast<size_t>((n0 + wn * 32) / 32) * (HT_ROWS * 64);
-  f32x16 acc[2][5];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 5; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-  tall_gemm_dispatch(rows, H / TK, wblk, tok0, ntb, acc);
+#endif
 
   const int r32 = lane & 31, kq = lane >> 5;
-  constexpr int SLD = 32 + 8;  // slab row stride, bf16 elements
-  unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * 32 * SLD;
+  unsigned char* slab = lds_raw;
+  if (!down) {
+    constexpr int LD = G1_COLS * 2 + 16;  // slab row pitch in bytes
 #pragma unroll
-  for (int j = 0; j < 5; ++j) {
-    if (j < ntb) {
+    for (int j = 0; j < JT; ++j)
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         float hv[4];
@@ -1225,118 +772,113 @@ __device__ __noinline__ void tall_gateup_task(ParamsRef pv, const TileDesc& tile
         uint2 pk;
         pk.x = pack_bf16(hv[0], hv[1]);
         pk.y = pack_bf16(hv[2], hv[3]);
-        *reinterpret_cast<uint2*>(slab + r32 * SLD + g4 * 8 + kq * 4) = pk;
+        *reinterpret_cast<uint2*>(slab + (j * 32 + r32) * LD + (wave * 32 + g4 * 8 + kq * 4) * 2) = pk;
       }
-      lds_wave_sync();
+    __syncthreads();
+    // 16 lanes store one row's 256 bytes; a wave stores 4 rows per instruction
+    unsigned char* h = uni(reinterpret_cast<unsigned char*>(p.h)) + (static_cast<size_t>(row0) * I + n0) * 2;
+    // (the reads of a batch first, then its stores: a store's assembly orders memory
+    // operations around it, and one LDS round trip per store would add up to microseconds)
+    constexpr int NIT = 8 * JT / WAVES, BATCH = 8;
 #pragma unroll
-      for (int b16 = 0; b16 < 2; ++b16) {
-        // one 1 KiB run: 16-row block b16 of this token block, chunk lane / 16 of row lane % 16
-        const int rr = b16 * 16 + (lane & 15), cc = (lane >> 4) * 8;
-        const int trow = tok0 + j * 32 + rr;
-        const uint4 v = *reinterpret_cast<const uint4*>(slab + rr * SLD + cc);
-        if (trow < tile.rows) st16_through(h + ((tok0 + j * 32) / 16 + b16) * 1024 + lane * 16, v);
+    for (int it0 = 0; it0 < NIT; it0 += BATCH) {
+      uint4 v[BATCH];
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        const int row = ((it0 + u) * WAVES + wave) * 4 + (lane >> 4);
+        if (it0 + u < NIT) v[u] = *reinterpret_cast<const uint4*>(slab + row * LD + (lane & 15) * 16);
       }
-      lds_wave_sync();
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        const int row = ((it0 + u) * WAVES + wave) * 4 + (lane >> 4);
+        if (it0 + u < NIT && row < rows)
+          st16_through(h + static_cast<size_t>(row) * I * 2 + (lane & 15) * 16, v[u]);
+      }
+    }
+    __syncthreads();  // the slab is stage memory again
+  } else {
+    int* sdst = reinterpret_cast<int*>(lds_raw + SIDE_OFF);
+    float* sw = reinterpret_cast<float*>(lds_raw + SIDE_OFF + TM_MAX * 4);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int r = static_cast<int>(threadIdx.x) + k * T_THREADS;
+      if (r < TM_MAX) {
+        sdst[r] = side_dst[k];
+        sw[r] = side_w[k];
+      }
+    }
+    __syncthreads();
+    unsigned char* y = uni(reinterpret_cast<unsigned char*>(p.y)) + n0 * 2;
+#pragma unroll
+    for (int part = 0; part < (JT + 3) / 4; ++part) {
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int j = part * 4 + jj;
+        if (j < JT) {
+          const float w = sw[j * 32 + r32];
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+              uint2 pk;
+              pk.x = pack_bf16(acc[i][j][g4 * 4 + 0] * w, acc[i][j][g4 * 4 + 1] * w);
+              pk.y = pack_bf16(acc[i][j][g4 * 4 + 2] * w, acc[i][j][g4 * 4 + 3] * w);
+              *reinterpret_cast<uint2*>(slab + (jj * 32 + r32) * EPI_LD +
+                                        (wave * 64 + i * 32 + g4 * 8 + kq * 4) * 2) = pk;
+            }
+        }
+      }
+      __syncthreads();
+      // 32 lanes store one row's 512 bytes at the row's (token, slot); a wave stores 2 rows per instruction
+      constexpr int BATCH = 8;
+#pragma unroll
+      for (int it0 = 0; it0 < 128 / (2 * WAVES); it0 += BATCH) {
+        uint4 v[BATCH];
+        int dst[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          const int lr = ((it0 + u) * WAVES + wave) * 2 + (lane >> 5);  // row inside this part
+          const int row = part * 128 + lr;
+          dst[u] = row < 32 * JT ? sdst[row] : -1;
+          v[u] = *reinterpret_cast<const uint4*>(slab + lr * EPI_LD + (lane & 31) * 16);
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+          if (dst[u] >= 0) st16_through(y + static_cast<size_t>(dst[u]) * H * 2 + (lane & 31) * 16, v[u]);
+      }
+      __syncthreads();
     }
   }
 }
 
-__device__ __noinline__ void tall_down_task(ParamsRef pv, const TileDesc& tile_in, int m, int nblk) {
+// one straight-line instantiation per number of live token blocks
+__device__ __noinline__ void tiled_gemm_task(ParamsRef pv, const TileDesc& tile_in, int nblk, int down_in,
+                                             unsigned* pend_in, unsigned* queue_in) {
   ParamsRef p = uniform_params(pv);
-  const int H = uni(p.H), I = uni(p.I);
-  TileDesc tile;
-  tile.expert = uni(tile_in.expert);
-  tile.row0 = uni(tile_in.row0);
-  tile.rows = uni(tile_in.rows);
-  const int n0 = uni(nblk) * TN;
-  const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const unsigned short* w2 = uni(reinterpret_cast<const unsigned short*>(p.ffn2)) +
-                             static_cast<size_t>(tile.expert) * H * I;
-  TallRows rows;
-  rows.tbase = uni(reinterpret_cast<const unsigned char*>(p.h)) + static_cast<size_t>(uni(m)) * tiled_h_tile_bytes(I);
-  rows.tkstride = static_cast<unsigned>(HT_ROWS * 64);
-  rows.tpacked = true;
-  rows.wpacked = uni(p.ffn2_packed != nullptr ? 1 : 0) != 0;
-  rows.wkstride = rows.wpacked ? 4096u : static_cast<unsigned>(TK * 2);
-#pragma unroll
-  for (int q = 0; q < LQ; ++q) {
-    const int row = stage_row(q);
-    if (rows.wpacked) {
-      const int B = wave * LQ + q;
-      const size_t task = static_cast<size_t>(tile.expert) * (H / 64) + (n0 / 64 + (B >> 2));
-      rows.wbase[q] = uni(reinterpret_cast<const unsigned char*>(p.ffn2_packed)) +
-                      task * (static_cast<size_t>(I / 32) * 4096) + (B & 3) * 1024;
-      rows.woff[q] = lane * 16;
-    } else {
-      rows.wbase[q] = reinterpret_cast<const unsigned char*>(w2);
-      rows.woff[q] = static_cast<unsigned>(n0 + row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
-    }
-  }
-#pragma unroll
-  for (int q = 0; q < 3; ++q) rows.toff[q] = static_cast<unsigned>(max(tall_token_block(q), 0) * 1024 + lane * 16);
-  const int wn = wave & 3, wm = wave >> 2;
-  const int wblk[2] = {wn * 64, wn * 64 + 32};
-  const int tok0 = wm * 160;
-  const int ntb = uni(min(5, (tile.rows - tok0 + 31) / 32));
-  const int r32 = lane & 31, kq = lane >> 5;
-  unsigned short* y = uni(reinterpret_cast<unsigned short*>(p.y)) + n0 + wn * 64 + (lane & 7) * 8;
-  float roww[5];
-  int dstrow[5];
-  {
-    const float* row_w = uni(p.row_w) + tile.row0;
-    const int* perm = uni(p.perm) + tile.row0;
-#pragma unroll
-    for (int j = 0; j < 5; ++j) {
-      const int myrow = tok0 + j * 32 + r32;
-      const bool valid = myrow < tile.rows;
-      roww[j] = valid ? ldc(&row_w[myrow]) : 0.0f;
-      dstrow[j] = valid ? ldc(&perm[myrow]) : -1;
-    }
-  }
-  f32x16 acc[2][5];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 5; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-  tall_gemm_dispatch(rows, I / TK, wblk, tok0, ntb, acc);
-
-  constexpr int SLD = 64 + 8;  // slab row stride, bf16 elements
-  unsigned short* slab = reinterpret_cast<unsigned short*>(lds_raw) + wave * (32 * SLD);
-#pragma unroll
-  for (int j = 0; j < 5; ++j) {
-    if (j < ntb) {
-      const float w = roww[j];
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          uint2 pk;
-          pk.x = pack_bf16(acc[i][j][g4 * 4 + 0] * w, acc[i][j][g4 * 4 + 1] * w);
-          pk.y = pack_bf16(acc[i][j][g4 * 4 + 2] * w, acc[i][j][g4 * 4 + 3] * w);
-          *reinterpret_cast<uint2*>(slab + r32 * SLD + i * 32 + g4 * 8 + kq * 4) = pk;
-        }
-      lds_wave_sync();
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        // eight lanes store one row's 128 bytes: rows 8*it .. 8*it+7
-        const int q = lane >> 3;
-        int dst = -1;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          const int d = __builtin_amdgcn_readlane(dstrow[j], it * 8 + r);
-          dst = q == r ? d : dst;
-        }
-        const uint4 v = *reinterpret_cast<const uint4*>(slab + (it * 8 + q) * SLD + (lane & 7) * 8);
-        if (dst >= 0) st16_through(y + static_cast<size_t>(dst) * H, v);
-      }
-      lds_wave_sync();
-    }
+  unsigned* pend = uni(pend_in);
+  unsigned* queue = uni(queue_in);
+  const int expert = uni(tile_in.expert), row0 = uni(tile_in.row0), rows = uni(tile_in.rows);
+  const bool down = uni(down_in) != 0;
+  const int jt = (rows + 31) >> 5;
+  if (jt > 9) {
+    if (down) tile_task<10, true>(p, expert, row0, rows, nblk, pend, queue); else tile_task<10, false>(p, expert, row0, rows, nblk, pend, queue);
+  } else if (jt > 8) {
+    if (down) tile_task<9, true>(p, expert, row0, rows, nblk, pend, queue); else tile_task<9, false>(p, expert, row0, rows, nblk, pend, queue);
+  } else if (jt > 7) {
+    if (down) tile_task<8, true>(p, expert, row0, rows, nblk, pend, queue); else tile_task<8, false>(p, expert, row0, rows, nblk, pend, queue);
+  } else if (jt > 6) {
+    if (down) tile_task<7, true>(p, expert, row0, rows, nblk, pend, queue); else tile_task<7, false>(p, expert, row0, rows, nblk, pend, queue);
+  } else if (jt > 4) {
+    if (down) tile_task<6, true>(p, expert, row0, rows, nblk, pend, queue); else tile_task<6, false>(p, expert, row0, rows, nblk, pend, queue);
+  } else if (jt > 2) {
+    if (down) tile_task<4, true>(p, expert, row0, rows, nblk, pend, queue); else tile_task<4, false>(p, expert, row0, rows, nblk, pend, queue);
+  } else {
+    if (down) tile_task<2, true>(p, expert, row0, rows, nblk, pend, queue); else tile_task<2, false>(p, expert, row0, rows, nblk, pend, queue);
   }
 }
 
+constexpr int TILED_LDS_BYTES =
+    NOTE_OFF + NOTE_BYTES > ROUTER_LDS_BYTES ? NOTE_OFF + NOTE_BYTES : ROUTER_LDS_BYTES;
 
 // combine: out[t] = sum over slots, in slot order, of y[t*K+slot]
 // (refFullMoe.h:35,62-65).
@@ -1391,7 +933,6 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
   }
   __syncthreads();  // flag[] is reused by the next task
 }
-
 // ---------------------------------------------------------------- worker loop
 // Ticket layout. The prologue (router, scan, scatter) uses one global counter.
 // The GEMM tasks are split into eight queues, one per XCD: queue x owns a
@@ -1423,9 +964,7 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
   Control* ctl = p.ctl;
   const unsigned T = static_cast<unsigned>(p.T);
   const unsigned n_sc = (T + RT_TOK - 1u) / RT_TOK;  // scatter tasks
-  // router tasks: of 16 tokens while every workgroup still gets at most one
-  const bool router16 = (T + RT16_TOK - 1u) / RT16_TOK <= gridDim.x;
-  const unsigned n_rt = router16 ? (T + RT16_TOK - 1u) / RT16_TOK : n_sc;
+  const unsigned n_rt = (T + RT16_TOK - 1u) / RT16_TOK;  // router tasks
   const unsigned n_es = (static_cast<unsigned>(p.E) + SCAN_EXPERTS - 1u) / SCAN_EXPERTS;
   const unsigned t_escan0 = n_rt;
   const unsigned t_scan = n_rt + n_es;
@@ -1446,7 +985,11 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
       st16(reinterpret_cast<char*>(r) + 16,
            u32x4{static_cast<unsigned>(t_fetch), static_cast<unsigned>(t_fetch >> 32),
                  static_cast<unsigned>(t_ready), static_cast<unsigned>(t_ready >> 32)});
+#ifdef FMOE_TRACE_PHASES
+      const unsigned x0 = task_notes()[1], x1 = task_notes()[2];
+#else
       const unsigned x0 = 0u, x1 = 0u;
+#endif
       st16(reinterpret_cast<char*>(r) + 32,
            u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), x0, x1});
     }
@@ -1464,11 +1007,7 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
     long long t_ready = 0;
     if (tk < n_rt) {
       if (p.trace) t_ready = wall_clock64();
-      if (router16) {
-        tiled_router16_task(p, static_cast<int>(tk));
-      } else {
-        tiled_router_task(p, static_cast<int>(tk));
-      }
+      tiled_router_task(p, static_cast<int>(tk));
       wg_arrive<false>(&ctl->router_done.v, &sh);
       trace(tk, 0, tk, t_fetch, t_ready);
     } else if (tk < t_scan) {
@@ -1510,12 +1049,25 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
     const unsigned lo = nm * q / 8u, hi = nm * (q + 1u) / 8u;
     const unsigned tiles = hi - lo;
     const unsigned q1 = tiles * nt1, q2 = tiles * nt2;
-    // the first ticket of a queue is drawn on its own, the others together with the
-    // arrival of the task before
+    // The first ticket of a queue is drawn on its own; every task then draws its successor
+    // while it runs, and its own completion is signalled under the next task (`pend`), so a
+    // workgroup goes from one task's last store to the next task's first load without a trip
+    // to memory. A completion that is still pending is signalled at once (after waiting for
+    // the stores) when the next task has to wait for a dependency or there is no next task:
+    // nobody may wait on a counter that a waiting workgroup holds back.
     if (threadIdx.x == 0) sh.ticket = add_relaxed(&ctl->xq[q].v, 1u);
     __syncthreads();
     unsigned j = sh.ticket;
     __syncthreads();
+    unsigned* pend = nullptr;
+    auto flush = [&]() {
+      if (pend != nullptr) {
+        fence_release();
+        __syncthreads();
+        if (threadIdx.x == 0) (void)add_relaxed(pend, 1u);
+        pend = nullptr;
+      }
+    };
     while (ok) {
       const long long t_fetch = p.trace ? wall_clock64() : 0;
       if (j >= q1 + q2) break;
@@ -1524,36 +1076,50 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
         const unsigned m = lo + j / nt1;
         if (p.trace) t_ready = wall_clock64();
         const TileDesc tile = ld_tile(&p.mtiles[m]);
-        if (tile.rows > TM) {
-          tall_gateup_task(p, tile, static_cast<int>(m), static_cast<int>(j % nt1));
-        } else {
-          tiled_gateup_task(p, tile, static_cast<int>(m), static_cast<int>(j % nt1));
-        }
-        const unsigned done = j;
-        wg_arrive_and_draw(&p.g1_done[m].v, &ctl->xq[q].v, j, &sh);
-        trace(t_dyn0 + lo * nt1 + done, 3, m, t_fetch, t_ready);
+#ifdef FMOE_X_SYNC
+        fence_release();
+        __syncthreads();
+#endif
+        tiled_gemm_task(p, tile, static_cast<int>(j % nt1), 0, pend, &ctl->xq[q].v);
+        pend = &p.g1_done[m].v;
+#ifdef FMOE_X_FLUSH
+        flush();
+#endif
+        trace(t_dyn0 + lo * nt1 + j, 3, m, t_fetch, t_ready);
+        j = task_notes()[0];
       } else {
         const unsigned jj = j - q1;
         const unsigned m = lo + jj / nt2;
         const TileDesc tile = ld_tile(&p.mtiles[m]);  // in flight while thread 0 looks at the counter
+        if (pend != nullptr) {
+          if (threadIdx.x == 0) sh.ok = ld_relaxed(&p.g1_done[m].v) >= nt1 ? 1u : 0u;
+          __syncthreads();
+          const bool ready = sh.ok != 0u;
+          __syncthreads();
+          if (!ready) flush();
+        }
         ok = wg_wait_ge(p, &p.g1_done[m].v, nt1, &sh);
         if (ok) {
           if (p.trace) t_ready = wall_clock64();
-          if (tile.rows > TM) {
-            tall_down_task(p, tile, static_cast<int>(m), static_cast<int>(jj % nt2));
-          } else {
-            tiled_down_task(p, tile, static_cast<int>(m), static_cast<int>(jj % nt2));
-          }
-          if (wg_arrive_and_draw(&ctl->g2_done.v, &ctl->xq[q].v, j, &sh) == n2_total - 1u)
-            wg_broadcast_flag(p, FLAG_G2);
+#ifdef FMOE_X_SYNC
+          fence_release();
+          __syncthreads();
+#endif
+          tiled_gemm_task(p, tile, static_cast<int>(jj % nt2), 1, pend, &ctl->xq[q].v);
+          pend = &ctl->g2_done.v;
+#ifdef FMOE_X_FLUSH
+          flush();
+#endif
           trace(t_dyn0 + nm * nt1 + lo * nt2 + jj, 4, m, t_fetch, t_ready);
+          j = task_notes()[0];
         }
       }
     }
+    flush();
   }
 
   // ---- combine tasks from the last global counter
-  if (ok && n2_total != 0u) ok = wg_wait_flag(p, FLAG_G2, &sh);
+  if (ok && n2_total != 0u) ok = wg_wait_ge(p, &ctl->g2_done.v, n2_total, &sh);
   while (ok) {
     const long long t_fetch = p.trace ? wall_clock64() : 0;
     if (threadIdx.x == 0) sh.ticket = add_relaxed(&ctl->cticket.v, 1u);
