@@ -56,7 +56,6 @@ C_ABI = {
                                       ctypes.POINTER(ctypes.c_uint), ctypes.c_void_p]),
     "flashMoeSetWaitLimitMs": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_double]),
     "flashMoeSchedFor": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
-    "flashMoeSetDenseSmallBatch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "flashMoeTraceEnable": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "flashMoeTraceRead": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint,
                                          ctypes.c_void_p]),

@@ -154,6 +154,28 @@ __device__ __forceinline__ void broadcast_flag(ParamsRef p, int which) {
   for (int g = lane_id(); g < n; g += 64) st_relaxed(&flags[g].f[which], 1u);
 }
 
+// A launch that raised an error bit (a bounded wait ran out, the tile table overflowed) has
+// left counters, masks and outputs in an arbitrary state. The last worker to leave makes
+// the failure visible and the launcher usable again without any help from the host, which
+// may be replaying a captured graph and never look: every element of `out` becomes NaN,
+// the workspace's zero region returns to zero (the count of completed launches apart), and
+// the bits are added to the launcher's word in pinned host memory, where the next Launch
+// finds them. `tid` of `nthreads` threads of that worker call this; nobody else is running.
+__device__ __forceinline__ void recover_after_error(ParamsRef p, unsigned err, int tid, int nthreads) {
+  unsigned* ws = reinterpret_cast<unsigned*>(p.ctl);
+  const unsigned launches_word =
+      static_cast<unsigned>(reinterpret_cast<unsigned*>(&p.ctl->launches.v) - ws);
+  const unsigned nz = p.zero_words;
+  for (unsigned i = tid; i < nz; i += nthreads)
+    if (i != launches_word) stc(&ws[i], 0u);
+  const size_t nout = static_cast<size_t>(p.T) * p.H * p.elem_bytes / 4;
+  const unsigned nan_word = p.elem_bytes == 2 ? 0x7FC07FC0u : 0x7FC00000u;
+  unsigned* out = reinterpret_cast<unsigned*>(p.out);
+  for (size_t i = tid; i < nout; i += nthreads) stc(&out[i], nan_word);
+  if (tid == 0 && p.host_error != nullptr)
+    __hip_atomic_fetch_or(as_global(p.host_error), err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // Wave-uniform bounded wait for *p >= target. False on time-out or when
 // another worker has raised an error; the caller then leaves the loop.
 __device__ __forceinline__ bool wave_wait_ge(const unsigned* p, unsigned target,

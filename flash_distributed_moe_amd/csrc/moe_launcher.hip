@@ -28,6 +28,8 @@ hipError_t pack_weights(const void* src, void* dst, int dtype, int E, int H, int
                         hipStream_t stream);
 hipError_t launch_tiled_kernel(const Params& p, int grid, hipStream_t stream);
 hipError_t prepare_tiled_kernel();
+hipError_t stream_kernel_occupancy(int dtype, int* per_cu);
+hipError_t tiled_kernel_occupancy(int* per_cu);
 int tiled_max_tokens();
 }
 
@@ -97,9 +99,8 @@ Layout make_layout(const FlashMoeLayerDesc& d, bool need_tiled) {
   L.perm = take(sizeof(int) * rows);
   L.row_w = take(sizeof(float) * rows);
   L.mtiles = take(sizeof(fmoe::TileDesc) * L.max_mtiles);
-  // h: [rows, I] routed, or [E, 64, I] when small batches run gate/up densely
-  (void)need_tiled;  // both variants keep h as [rows, I]
-  const size_t h_rows = std::max<size_t>(rows, static_cast<size_t>(d.experts) * 64);
+  (void)need_tiled;  // both variants keep h as [rows, I], rows in permuted order
+  const size_t h_rows = rows;
   L.h = take(esz * h_rows * d.intermediate);
   L.y = take(sizeof(float) * rows * d.hidden);
   const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
@@ -177,13 +178,13 @@ struct FlashMoeLauncher {
   long long ticks_per_ms = 100000;
   long long spin_limit = 0;
   int last_tokens = 0;
-  // Batches of at most 16 tokens may run gate/up for every (expert, token) pair
-  // without waiting for the routing. Off unless asked for: it reads every
-  // expert's gate/up weights, which measured slower than the routed path at
-  // every batch size (T=1: 199 vs 88 us, T=16: 250 vs 231 us on the 30B shape).
-  bool dense_ok = false;
   fmoe::TraceRec* trace = nullptr;
   unsigned trace_cap = 0;
+  // One word of pinned host memory that a failing launch's last worker adds its error
+  // bits to (null for the launcher-less entry point, which may not allocate).
+  unsigned reported_error = 0;         // bits Launch has reported since the last flashMoeStatus
+  unsigned* host_error = nullptr;      // host address
+  unsigned* host_error_dev = nullptr;  // the same word as the device addresses it
 };
 
 namespace {
@@ -201,10 +202,6 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.n_groups = l->num_cus < kMaxGroups ? l->num_cus : kMaxGroups;
   p.n_workers = p.n_groups * 8;
   p.fuse_scatter = (static_cast<long long>(T) * d.top_k <= 2048) ? 1 : 0;
-  // Dense gate/up re-reads every token row for every expert; measured on MI355X
-  // it pays while one 16-row MFMA block holds the whole batch and costs more
-  // than the hidden routing prologue beyond that.
-  p.dense = (T <= 16 && l->dense_ok) ? 1 : 0;
   // Early gate/up tasks wait inside the kernel for the routing, so every routing
   // task must be among the tickets the workers start with: they go to the first
   // workgroups, four dot tasks and four select/scan tasks each (half of the
@@ -232,13 +229,12 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   // 242 / 253, T=192 263 / 266), two up to 24.
   const long long slots = static_cast<long long>(T) * d.top_k;
   const int early_blocks = slots <= 12ll * d.experts ? 1 : slots <= 24ll * d.experts ? 2 : 0;
-  p.early = (reaches_experts && early_blocks != 0 && !p.dense && p.fuse_scatter &&
+  p.early = (reaches_experts && early_blocks != 0 && p.fuse_scatter &&
              T <= fmoe::EARLY_MAX_TOKENS &&
              d.experts * ((T + 63) / 64) <= fmoe::SCAN_LDS_WORDS && d.experts <= L.max_mtiles &&
              routing_groups <= p.n_groups / 2)
                 ? early_blocks
                 : 0;
-  p.tpad = (T + 15) / 16 * 16;
   p.max_mtiles = L.max_mtiles;
   p.spin_limit = l->spin_limit;
   p.tokens = tokens;
@@ -267,6 +263,9 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.mtiles = reinterpret_cast<fmoe::TileDesc*>(w + L.mtiles);
   p.h = w + L.h;
   p.y = reinterpret_cast<float*>(w + L.y);
+  p.host_error = l->host_error_dev;
+  p.zero_words = static_cast<unsigned>(L.zero_bytes / 4);
+  p.elem_bytes = d.dtype == FLASH_MOE_BF16 ? 2 : 4;
   p.trace = l->trace;
   p.trace_cap = l->trace_cap;
   return p;
@@ -314,6 +313,7 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
 
   auto fail = [&](hipError_t e) {
     if (l->ws) (void)hipFree(l->ws);
+    if (l->host_error) (void)hipHostFree(l->host_error);
     delete l;
     printf("[MOE HIP ERROR: %s]: create failed: %s\n", FMOE_FILENAME, hipGetErrorString(e));
     return static_cast<int>(e);
@@ -330,7 +330,21 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
   l->spin_limit = 2000 * l->ticks_per_ms;
   if ((e = fmoe::prepare_stream_kernel()) != hipSuccess) return fail(e);
   if ((e = fmoe::prepare_tiled_kernel()) != hipSuccess) return fail(e);
+  // Waits happen inside the kernels, so every workgroup of a launch must be resident at
+  // once: one per CU, which both kernels' resources allow only if nothing else is asked of them.
+  int per_cu = 0;
+  if ((e = fmoe::stream_kernel_occupancy(desc->dtype, &per_cu)) != hipSuccess) return fail(e);
+  if (per_cu < 1) return fail(hipErrorLaunchOutOfResources);
+  if ((e = fmoe::tiled_kernel_occupancy(&per_cu)) != hipSuccess) return fail(e);
+  if (per_cu < 1) return fail(hipErrorLaunchOutOfResources);
   if ((e = hipMalloc(reinterpret_cast<void**>(&l->ws), l->layout.total)) != hipSuccess)
+    return fail(e);
+  if ((e = hipHostMalloc(reinterpret_cast<void**>(&l->host_error), 64, hipHostMallocDefault)) !=
+      hipSuccess)
+    return fail(e);
+  *l->host_error = 0u;
+  if ((e = hipHostGetDevicePointer(reinterpret_cast<void**>(&l->host_error_dev), l->host_error,
+                                   0)) != hipSuccess)
     return fail(e);
   if ((e = hipMemsetAsync(l->ws, 0, l->layout.zero_bytes, stream)) != hipSuccess) return fail(e);
   if (desc->flags & FLASH_MOE_FLAG_PACK_WEIGHTS) {
@@ -355,6 +369,19 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
   if (tokens_num > l->desc.max_tokens)
     FMOE_FAIL(hipErrorUnknown, "tokens_num = %i exceeds max_tokens = %i", tokens_num,
               l->desc.max_tokens);
+  // A launch that failed on the device (see flashMoeStatus for the bits) has left NaN in its
+  // output and the launcher ready for use; the first Launch after it has finished reports it.
+  if (l->host_error != nullptr) {
+    const unsigned bits = *static_cast<volatile unsigned*>(l->host_error);
+    if (bits != 0u) {
+      *static_cast<volatile unsigned*>(l->host_error) = 0u;
+      l->reported_error |= bits;
+      FMOE_FAIL(hipErrorUnknown,
+                "an earlier launch failed on the device (error bits 0x%x: 1 = a dependency wait "
+                "ran out, 2 = row-tile table overflow); its output is NaN; nothing was launched now",
+                bits);
+    }
+  }
   if (tokens_num == 0) return hipSuccess;
   if (tokens == nullptr || output == nullptr)
     FMOE_FAIL(hipErrorInvalidValue, "null tokens/output pointer");
@@ -490,6 +517,7 @@ int flashMoeDestroy(FlashMoeLauncher* l, void* stream_) {
   if (l == nullptr) return hipSuccess;
   FMOE_HIP_CHECK(hipStreamSynchronize(stream));
   FMOE_HIP_CHECK(hipFree(l->ws));
+  if (l->host_error) FMOE_HIP_CHECK(hipHostFree(l->host_error));
   if (l->trace) FMOE_HIP_CHECK(hipFree(l->trace));
   delete l;
   return hipSuccess;
@@ -527,7 +555,13 @@ int flashMoeStatus(FlashMoeLauncher* l, unsigned* error_bits, unsigned* launches
   FMOE_HIP_CHECK(hipStreamSynchronize(stream));
   fmoe::Control c;
   FMOE_HIP_CHECK(hipMemcpy(&c, l->ws + l->layout.ctl, sizeof(c), hipMemcpyDeviceToHost));
-  if (error_bits) *error_bits = c.error.v;
+  unsigned bits = c.error.v | l->reported_error;
+  l->reported_error = 0u;
+  if (l->host_error != nullptr) {
+    bits |= *static_cast<volatile unsigned*>(l->host_error);
+    *static_cast<volatile unsigned*>(l->host_error) = 0u;
+  }
+  if (error_bits) *error_bits = bits;
   if (launches) *launches = c.launches.v;
   if (c.error.v != 0u) {
     // an aborted launch leaves counters and masks in an arbitrary state
@@ -561,12 +595,6 @@ int flashMoeTraceRead(FlashMoeLauncher* l, void* records, unsigned max_records, 
   FMOE_HIP_CHECK(hipMemcpy(records, l->trace, sizeof(fmoe::TraceRec) * static_cast<size_t>(n),
                            hipMemcpyDeviceToHost));
   FMOE_HIP_CHECK(hipMemset(l->trace, 0xFF, sizeof(fmoe::TraceRec) * static_cast<size_t>(l->trace_cap)));
-  return hipSuccess;
-}
-
-int flashMoeSetDenseSmallBatch(FlashMoeLauncher* l, int enable) {
-  if (l == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher");
-  l->dense_ok = enable != 0;
   return hipSuccess;
 }
 

@@ -123,12 +123,17 @@ struct Params {
   unsigned* tok_arrive;            // [T] expert groups of the token whose keys are in
   int n_groups;                    // workgroups in the grid
   int fuse_scatter;                // 1: the scan task also writes the permutation
-  int dense;                       // 1: gate/up runs for every (expert, token) pair (small batches)
   int early;                       // 1, 2: row tile e belongs to expert e (empty or not), so gate/up tasks are
                                    //    handed out at launch and fetch their first weights under the routing
-  int tpad;                        // dense mode: h rows reserved per expert
   int dot16;                       // 1 (streaming variant, bf16): the logit chains run on the matrix core, 16 tokens x
                                    //    16 experts per workgroup, on the first workgroups before they take tickets
+  // What the last worker out needs when a launch has raised an error bit: it fills `out`
+  // with NaN, returns the workspace's leading zero_words 32-bit words (counters, flags,
+  // masks; `ctl` is the workspace's first byte) to zero, and adds the bits to *host_error
+  // (pinned host memory the host reads without waiting for the stream; may be null).
+  unsigned* host_error;
+  unsigned zero_words;
+  int elem_bytes;     // of tokens / out: 2 or 4
   TraceRec* trace;    // null unless tracing; indexed by ticket
   unsigned trace_cap;
 };

@@ -17,13 +17,6 @@
 // The down projection reads h rows that other workers wrote, so its B operand
 // uses coherent loads.
 //
-// Batches of at most 16 tokens run gate/up "dense": every expert is applied to
-// every token (h is [expert][token][I]), which makes the gate/up tasks
-// independent of the router: they start streaming at once and the routing
-// prologue hides behind them. (The code handles up to 64 tokens that way, but
-// beyond one 16-row MFMA block the extra token-row loads cost more bandwidth
-// than the hidden prologue is worth.)
-//
 // Replaces, for this regime, the reference's moeKernel
 // (src/hip/kernel/moeKernel.h:37-107), its task executors
 // (src/hip/kernel/tasks/*.h) and its queue (src/hip/taskSystem/*.h).
@@ -691,7 +684,6 @@ struct RoundSteps {
 // h[row, n0 .. n0+16*G1_NB) for the rows of one tile. Follows
 // refExpertFFN1.h:51-65 (two GEMMs against the [2I,H] expert matrix, then
 // SiLU(gate) * up), accumulated on MFMA in float.
-// DENSE: the tile is (expert, all tokens): row r is token r, h row = row0 + r.
 // The row tile of expert e read off the top-k table alone: its rows are the
 // entries i = token*K + slot that name e, in ascending i (the order the
 // permutation gives them), and its first row is the number of entries that name
@@ -757,7 +749,7 @@ __device__ __forceinline__ void tile_from_topk(ParamsRef p, int e, int& row0, in
 // Returns 0: done (or the tile is empty), 1: the wait failed, 2 (EARLY only):
 // the tile has more than 16*RB rows, nothing was written, and the caller runs
 // the task again from the tile table with more row blocks.
-template <typename DT, int RB, bool DENSE, bool EARLY>
+template <typename DT, int RB, bool EARLY>
 __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk,
                                            unsigned* lds_flag, unsigned* lds_poller) {
   typedef typename DT::elem elem;
@@ -792,7 +784,7 @@ __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       const int row = min(r * 16 + r16, tile.rows - 1);
-      const int tok = DENSE ? row : ldc(&p.perm[tile.row0 + row]) / p.K;
+      const int tok = ldc(&p.perm[tile.row0 + row]) / p.K;
       bp[r] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(tok) * p.H + g * EPV;
     }
   };
@@ -851,7 +843,7 @@ __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk
   return 0;
 }
 
-template <typename DT, int RB, bool DENSE>
+template <typename DT, int RB>
 __device__ __noinline__ void gateup_task(ParamsRef pv, int expert, int row0, int rows, int nblk) {
   // (the row tile arrives as three integers: a struct by value makes the callee save
   // and restore every callee-saved register it touches, a struct by reference costs
@@ -862,7 +854,7 @@ __device__ __noinline__ void gateup_task(ParamsRef pv, int expert, int row0, int
   tile.row0 = row0;
   tile.rows = rows;
   tile.pad = 0;
-  gateup_body<DT, RB, DENSE, false>(p, tile, nblk, nullptr, nullptr);
+  gateup_body<DT, RB, false>(p, tile, nblk, nullptr, nullptr);
 }
 
 // the rows of the expert's tile are worked out inside, once the routing is known
@@ -875,7 +867,7 @@ __device__ __noinline__ int gateup_early_task(ParamsRef pv, int expert, int nblk
   tile.row0 = 0;
   tile.rows = 0;
   tile.pad = 0;
-  return gateup_body<DT, RB, false, true>(p, tile, nblk, lds_flag, lds_poller);
+  return gateup_body<DT, RB, true>(p, tile, nblk, lds_flag, lds_poller);
 }
 
 // ----------------------------------------------------------------------- down
@@ -884,7 +876,7 @@ __device__ __noinline__ int gateup_early_task(ParamsRef pv, int expert, int nblk
 // does (src/hip/kernel/tasks/ffn2Task.h:37-40). The weight rows do not depend
 // on h, so their first loads are issued before the wait for the tile's
 // gate/up tasks. Returns false if that wait failed.
-template <typename DT, int RB, bool DENSE>
+template <typename DT, int RB>
 __device__ __noinline__ bool down_task(ParamsRef pv, int expert, int row0, int rows, int nblk,
                                        unsigned* dep, unsigned dep_target) {
   ParamsRef p = uniform_params(pv);
@@ -918,18 +910,15 @@ __device__ __noinline__ bool down_task(ParamsRef pv, int expert, int row0, int r
       ap[b] = w2 + static_cast<size_t>(n0 + 16 * b + r16) * p.I + g * EPV;
   }
   // the part of h this tile reads (uniform; the offsets inside it fit 32 bits)
-  const size_t hrow0 = DENSE ? static_cast<size_t>(tile.expert) * p.tpad : static_cast<size_t>(tile.row0);
+  const size_t hrow0 = static_cast<size_t>(tile.row0);
   const elem* hbase = uniform_ptr(reinterpret_cast<const elem*>(p.h) + hrow0 * p.I);
   const unsigned hbytes = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(
-      (DENSE ? p.tpad : tile.rows) * p.I * static_cast<int>(sizeof(elem))));
+      tile.rows * p.I * static_cast<int>(sizeof(elem))));
   const elem* bp[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
     const int row = min(r * 16 + r16, tile.rows - 1);
-    // dense mode: h is [expert][tpad][I] and the row is the token's
-    const size_t hrow = DENSE ? static_cast<size_t>(tile.expert) * p.tpad +
-                                    ldc(&p.perm[tile.row0 + row]) / p.K
-                              : static_cast<size_t>(tile.row0 + row);
+    const size_t hrow = static_cast<size_t>(tile.row0 + row);
     bp[r] = reinterpret_cast<const elem*>(p.h) + hrow * p.I + g * EPV;
   }
   // gate weight and destination of this lane's rows: fetched now, so that their
@@ -1087,11 +1076,7 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
   const unsigned t_scan = n_router;
   const unsigned t_scatter0 = n_router + 1u;
   const unsigned nt1 = static_cast<unsigned>(p.I / (16 * G1_NB));
-  // dense mode: one gate/up task per (expert, column block), known at launch,
-  // ticketed right after the routing prologue
-  const bool dense = p.dense != 0;
-  const unsigned t_dense0 = t_scatter0 + (p.fuse_scatter ? 0u : T);
-  const unsigned t_dyn0 = t_dense0 + (dense ? static_cast<unsigned>(p.E) * nt1 : 0u);
+  const unsigned t_dyn0 = t_scatter0 + (p.fuse_scatter ? 0u : T);
   const unsigned nt2 = static_cast<unsigned>(p.H / (16 * G2_NB));
   const unsigned ncomb = static_cast<unsigned>((p.H + COMBINE_COLS - 1) / COMBINE_COLS);
   const unsigned worker = blockIdx.x * waves_per_group + wave_in_group;
@@ -1195,36 +1180,17 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
       } else {
         scan_task(p);
       }
-    } else if (tk < t_dense0) {
+    } else if (tk < t_dyn0) {
       kind = 2;
       aux = tk - t_scatter0;
       if (!wait_flag(p, FLAG_SCAN, lds_flag, lds_poller)) break;
       if (p.trace) t_ready = wall_clock64();
       scatter_task(p, static_cast<int>(aux));
-    } else if (tk < t_dyn0) {
-      kind = 3;
-      const unsigned j = tk - t_dense0;
-      aux = j / nt1;  // expert
-      if (p.trace) t_ready = wall_clock64();
-      TileDesc tile;
-      tile.expert = static_cast<int>(aux);
-      tile.row0 = static_cast<int>(aux) * p.tpad;
-      tile.rows = p.T;
-      tile.pad = 0;
-      const int nblk = static_cast<int>(j % nt1);
-      if (p.T <= 16) {
-        gateup_task<DT, 1, true>(p, tile.expert, tile.row0, tile.rows, nblk);
-      } else if (p.T <= 32) {
-        gateup_task<DT, 2, true>(p, tile.expert, tile.row0, tile.rows, nblk);
-      } else {
-        gateup_task<DT, 4, true>(p, tile.expert, tile.row0, tile.rows, nblk);
-      }
-      wave_arrive(&p.g1_done[aux].v);
     } else {
       if (!have_dyn) {
         if (!wait_flag(p, FLAG_SCAN, lds_flag, lds_poller)) break;
         const unsigned nm = ldc(&ctl->n_mtiles.v);
-        n1 = dense ? 0u : nm * nt1;
+        n1 = nm * nt1;
         n2 = nm * nt2;
         nc = T * ncomb;
         have_dyn = true;
@@ -1254,11 +1220,11 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
           for (int r0 = 0; r0 < tile.rows; r0 += SKINNY_MT) {
             const int rc = min(SKINNY_MT, tile.rows - r0);
             if (rc <= 16) {
-              gateup_task<DT, 1, false>(p, tile.expert, tile.row0 + r0, rc, nblk);
+              gateup_task<DT, 1>(p, tile.expert, tile.row0 + r0, rc, nblk);
             } else if (rc <= 32) {
-              gateup_task<DT, 2, false>(p, tile.expert, tile.row0 + r0, rc, nblk);
+              gateup_task<DT, 2>(p, tile.expert, tile.row0 + r0, rc, nblk);
             } else {
-              gateup_task<DT, 4, false>(p, tile.expert, tile.row0 + r0, rc, nblk);
+              gateup_task<DT, 4>(p, tile.expert, tile.row0 + r0, rc, nblk);
             }
           }
         }
@@ -1274,11 +1240,11 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
         const TileDesc tile = ld_tile(&p.mtiles[aux]);
         const int nblk = static_cast<int>(j % nt1);
         if (tile.rows <= 16) {
-          gateup_task<DT, 1, false>(p, tile.expert, tile.row0, tile.rows, nblk);
+          gateup_task<DT, 1>(p, tile.expert, tile.row0, tile.rows, nblk);
         } else if (tile.rows <= 32) {
-          gateup_task<DT, 2, false>(p, tile.expert, tile.row0, tile.rows, nblk);
+          gateup_task<DT, 2>(p, tile.expert, tile.row0, tile.rows, nblk);
         } else {
-          gateup_task<DT, 4, false>(p, tile.expert, tile.row0, tile.rows, nblk);
+          gateup_task<DT, 4>(p, tile.expert, tile.row0, tile.rows, nblk);
         }
         wave_arrive(&p.g1_done[aux].v);
       } else if (j < n1 + n2) {
@@ -1292,22 +1258,7 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
         if (p.trace) t_ready = wall_clock64();
         const TileDesc tile = ld_tile(&p.mtiles[aux]);
         bool ok;
-        if (dense) {
-          // the expert's gate/up tasks are counted per expert; an expert has one
-          // row tile here (at most 64 rows); the permutation must be final too
-          if (!perm_ready) {
-            if (!wait_flag(p, FLAG_PERM, lds_flag, lds_poller)) break;
-            perm_ready = true;
-          }
-          unsigned* dep = &p.g1_done[tile.expert].v;
-          if (tile.rows <= 16) {
-            ok = down_task<DT, 1, true>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
-          } else if (tile.rows <= 32) {
-            ok = down_task<DT, 2, true>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
-          } else {
-            ok = down_task<DT, 4, true>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
-          }
-        } else {
+        {
           // the task reads its rows' gate weights and destinations up front
           if (!perm_ready) {
             if (!wait_flag(p, FLAG_PERM, lds_flag, lds_poller)) break;
@@ -1319,21 +1270,21 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
           if (tile.rows == 0) {
             ok = true;
           } else if (tile.rows <= 16) {
-            ok = down_task<DT, 1, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
+            ok = down_task<DT, 1>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           } else if (tile.rows <= 32) {
-            ok = down_task<DT, 2, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
+            ok = down_task<DT, 2>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           } else if (tile.rows <= SKINNY_MT) {
-            ok = down_task<DT, 4, false>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
+            ok = down_task<DT, 4>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
           } else {
             ok = true;
             for (int r0 = 0; ok && r0 < tile.rows; r0 += SKINNY_MT) {
               const int rc = min(SKINNY_MT, tile.rows - r0);
               if (rc <= 16) {
-                ok = down_task<DT, 1, false>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+                ok = down_task<DT, 1>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
               } else if (rc <= 32) {
-                ok = down_task<DT, 2, false>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+                ok = down_task<DT, 2>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
               } else {
-                ok = down_task<DT, 4, false>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+                ok = down_task<DT, 4>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
               }
             }
           }
@@ -1378,10 +1329,11 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
   }
   last = __builtin_amdgcn_readfirstlane(last);
   if (last) {
+    const unsigned err = ldc(&ctl->error.v);
+    if (err != 0u) recover_after_error(p, err, lane, 64);
     // (early mode: one row tile per expert, known without a trip to memory)
     unsigned nm = p.early ? static_cast<unsigned>(p.E)
                           : min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
-    if (dense) nm = max(nm, static_cast<unsigned>(p.E));  // counters are per expert there
     for (unsigned i = lane; i < nm; i += 64) stc(&p.g1_done[i].v, 0u);
     for (int g = lane; g < p.n_groups; g += 64) {
       stc(&p.wgflags[g].f[FLAG_SCAN], 0u);
@@ -1472,6 +1424,13 @@ hipError_t prepare_stream_kernel() {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(moe_stream_kernel<F32>),
                              hipFuncAttributeMaxDynamicSharedMemorySize,
                              static_cast<int>(max_lds));
+}
+
+hipError_t stream_kernel_occupancy(int dtype, int* per_cu) {
+  const size_t lds = static_cast<size_t>(8) * ROUTER_LDS_FLOATS * sizeof(float);
+  return dtype == DT_BF16
+             ? hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, moe_stream_kernel<BF16>, 512, lds)
+             : hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, moe_stream_kernel<F32>, 512, lds);
 }
 
 }  // namespace fmoe

@@ -1137,6 +1137,11 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
   if (threadIdx.x == 0) sh.ok = (add_relaxed(&ctl->exit_count.v, 1u) == n_groups - 1u) ? 1u : 0u;
   __syncthreads();
   if (sh.ok) {
+    const unsigned err = ldc(&ctl->error.v);
+    if (err != 0u) {
+      recover_after_error(p, err, static_cast<int>(threadIdx.x), T_THREADS);
+      __syncthreads();
+    }
     const unsigned nmr = min(ldc(&ctl->n_mtiles.v), static_cast<unsigned>(p.max_mtiles));
     for (unsigned i = threadIdx.x; i < nmr; i += T_THREADS) stc(&p.g1_done[i].v, 0u);
     for (unsigned g = threadIdx.x; g < n_groups; g += T_THREADS) {
@@ -1170,6 +1175,10 @@ hipError_t launch_tiled_kernel(const Params& p, int grid, hipStream_t stream) {
 hipError_t prepare_tiled_kernel() {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(moe_tiled_kernel),
                              hipFuncAttributeMaxDynamicSharedMemorySize, TILED_LDS_BYTES);
+}
+
+hipError_t tiled_kernel_occupancy(int* per_cu) {
+  return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, moe_tiled_kernel, T_THREADS, TILED_LDS_BYTES);
 }
 
 }  // namespace fmoe

@@ -179,9 +179,5 @@ class MoeKernelLauncher:
             _hip_check(self._lib.flashMoeRefreshWeights(self._h, _stream()),
                        "flashMoeRefreshWeights")
 
-    def set_dense_small_batch(self, enable):
-        _hip_check(self._lib.flashMoeSetDenseSmallBatch(self._h, 1 if enable else 0),
-                   "flashMoeSetDenseSmallBatch")
-
     def sched_for(self, tokens_num):
         return self._lib.flashMoeSchedFor(self._h, int(tokens_num))

@@ -82,8 +82,10 @@ int flashMoeRefreshWeights(FlashMoeLauncher* l, void* stream);
 
 /* Enqueues one forward pass on `stream` and returns without waiting.
  * tokens, output: device [tokens_num, H] in the layer dtype; output may alias
- * tokens. Launches on one launcher must be ordered on one stream.
- * hipErrorUnknown when tokens_num > max_tokens. */
+ * tokens. Launches on one launcher must be ordered on one stream (its waits
+ * happen inside the kernel, against its own workspace).
+ * hipErrorUnknown when tokens_num > max_tokens, or when an earlier launch failed
+ * on the device (see flashMoeStatus): then nothing is enqueued. */
 int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int tokens_num,
                    void* stream);
 
@@ -122,10 +124,17 @@ int flashMoeDestroy(FlashMoeLauncher* l, void* stream);
 int flashMoeReadRouting(FlashMoeLauncher* l, int tokens_num, int* topk_idx, float* topk_w,
                         int* expert_counts, int* expert_offsets, int* perm, void* stream);
 
-/* Waits for `stream`, reports the device error bits (1 = a dependency wait
- * timed out, 2 = tile table overflow) and the number of completed launches.
- * If error bits are set the launcher's counters are cleared so that it can be
- * used again. */
+/* Device-side failures. A dependency wait inside the kernel is bounded (see
+ * flashMoeSetWaitLimitMs); when one runs out, or the row-tile table overflows,
+ * the launch ends normally, its last worker fills the launch's output with NaN,
+ * returns the workspace to its initial state (so later launches and graph
+ * replays work) and adds the error bits to a word in pinned host memory. The
+ * first flashMoeLaunch made after that kernel has finished launches nothing and
+ * returns hipErrorUnknown (the reference aborts in a device assert instead,
+ * src/hip/utils/hipDeviceUtils.h:12); the launch after it runs normally.
+ * flashMoeStatus waits for `stream`, reports the bits raised since it was last
+ * called (1 = a dependency wait timed out, 2 = tile table overflow), including
+ * those a Launch has already reported, and the number of completed launches. */
 int flashMoeStatus(FlashMoeLauncher* l, unsigned* error_bits, unsigned* launches, void* stream);
 
 /* Bound on a single dependency wait inside the kernel, in milliseconds
@@ -144,12 +153,6 @@ int flashMoeSetWaitLimitMs(FlashMoeLauncher* l, double ms);
  * max_records records to the host and marks all records unused (all bits set). */
 int flashMoeTraceEnable(FlashMoeLauncher* l, unsigned capacity);
 int flashMoeTraceRead(FlashMoeLauncher* l, void* records, unsigned max_records, void* stream);
-
-/* 1: batches of at most 16 tokens run the gate/up projection for every (expert,
- * token) pair, so that it does not wait for the router. Default 0: gate/up runs
- * only for routed rows, after the router, which measured faster at every batch
- * size. Results are identical either way. No counterpart in the reference. */
-int flashMoeSetDenseSmallBatch(FlashMoeLauncher* l, int enable);
 
 /* Which scheduling variant a launch of tokens_num tokens would use. */
 int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num);

@@ -99,17 +99,18 @@ def test_nan_and_all_equal_logits(name):
 @pytest.mark.parametrize("name,T,sched", [("qwen3_30b_decode", 64, 1), ("qwen3_30b_decode", 512, 2)])
 def test_device_wait_limit_is_reported_and_cleared(name, T, sched):
     """With a wait limit of 100 ns every dependency wait that has to wait at all
-    gives up: the kernel ends normally, flashMoeStatus reports bit 1 and re-arms
-    the launcher, and the next launch with the normal limit is correct again."""
+    gives up: the kernel ends normally with NaN in its output, flashMoeStatus
+    reports bit 1, and the next launch with the normal limit is correct again."""
     cfg = synth.CONFIGS[name].replace(T=T, name="timeout")
     case = GpuCase(cfg, sched=sched)
     try:
         x = case.inp["tokens"]
         good = case.run().clone()
         case.launcher.set_wait_limit_ms(1e-4)
-        out = torch.empty_like(x)
+        out = torch.zeros_like(x)
         case.launcher.launch(x, out)
         torch.cuda.synchronize()
+        assert bool(torch.isnan(out).all()), "a failed launch must leave NaN in every output element"
         err, _ = case.launcher.status()
         assert err & 1, "the shortened wait did not time out"
         assert case.launcher.status()[0] == 0, "status must clear the error"
@@ -117,5 +118,38 @@ def test_device_wait_limit_is_reported_and_cleared(name, T, sched):
         again = case.run()
         assert torch.equal(again, good)
         case.check_outputs(x, again)
+    finally:
+        case.close()
+
+
+@pytest.mark.parametrize("name,T,sched", [("qwen3_30b_decode", 64, 1),
+                                          ("qwen3_30b_decode", 700, 2)])
+def test_device_failure_reaches_a_caller_that_never_asks(name, T, sched, capfd):
+    """A caller written against the reference's interface only ever calls Launch:
+    after a launch has failed on the device, the next Launch returns
+    hipErrorUnknown (nothing is launched), and the one after that is correct,
+    with no call of flashMoeStatus in between. A captured graph keeps working too."""
+    cfg = synth.CONFIGS[name].replace(T=T, name="timeout")
+    case = GpuCase(cfg, sched=sched)
+    try:
+        x = case.inp["tokens"]
+        good = case.run().clone()
+        case.launcher.set_wait_limit_ms(1e-4)
+        out = torch.zeros_like(x)
+        case.launcher.launch(x, out)            # fails on the device; Launch itself has returned success
+        torch.cuda.synchronize()
+        case.launcher.set_wait_limit_ms(2000.0)
+        untouched = torch.full_like(x, 3.0)
+        with pytest.raises(RuntimeError, match="hipError_t 999"):
+            case.launcher.launch(x, untouched)
+        torch.cuda.synchronize()
+        assert "an earlier launch failed on the device" in capfd.readouterr().out
+        assert bool((untouched == 3.0).all())   # nothing was launched
+        again = torch.empty_like(x)
+        case.launcher.launch(x, again)          # the launcher re-armed itself on the device
+        torch.cuda.synchronize()
+        assert torch.equal(again, good)
+        assert case.launcher.status()[0] & 1    # the bits are still there for whoever asks
+        assert case.launcher.status()[0] == 0
     finally:
         case.close()

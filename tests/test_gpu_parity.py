@@ -196,27 +196,6 @@ def test_tiled_variant_forced(shape):
         case.close()
 
 
-@pytest.mark.parametrize("T", [1, 5, 16])
-def test_dense_small_batch_equals_routed(T):
-    """On request, batches of <= 16 tokens run gate/up for every (expert, token)
-    pair; the routed path (the default) must give the same bits."""
-    cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=T, name="dense")
-    case = GpuCase(cfg, seed=40 + T)
-    try:
-        x = case.inp["tokens"]
-        case.launcher.set_dense_small_batch(True)
-        dense = case.run()
-        case.check_routing(x, case.launcher.routing(T))
-        case.check_outputs(x, dense)
-        case.launcher.set_dense_small_batch(False)
-        routed = case.run()
-        assert torch.equal(dense, routed)
-        case.launcher.set_dense_small_batch(True)
-        assert torch.equal(case.run(), dense)
-    finally:
-        case.close()
-
-
 @pytest.mark.parametrize("name,T", [("qwen3_30b_decode", 64), ("qwen3_30b_decode", 100),
                                     ("tiny_f32", 16)])
 def test_packed_weights_equal_unpacked(name, T):
