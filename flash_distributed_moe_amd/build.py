@@ -57,5 +57,41 @@ def build(verbose=True):
     return LIB_PATH
 
 
+PY_SRC = os.path.join(CSRC, "py", "flashMoeLauncherModule.cpp")
+ROOT = os.path.dirname(HERE)
+
+
+def py_extension_path():
+    import sysconfig
+
+    return os.path.join(ROOT, "flashMoeLauncher" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_py_extension(verbose=True):
+    """The `flashMoeLauncher` Python extension (pybind11 over the C++ interface), next to the
+    package so that `import flashMoeLauncher` finds it with the repository root on sys.path.
+    Host code only: compiled with g++ against torch's headers."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    out = py_extension_path()
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I" + sysconfig.get_paths()["include"]]
+    cmd += ["-I" + p for p in cpp_extension.include_paths()] + ["-I/opt/rocm/include"]
+    cmd += [PY_SRC, "-o", out, "-L" + tlib, "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_hip",
+            "-lc10_hip", "-ltorch_python", "-L" + LIB_DIR, "-lflashMoe", "-L/opt/rocm/lib",
+            "-lamdhip64", "-Wl,-rpath,$ORIGIN/flash_distributed_moe_amd/lib", "-Wl,-rpath," + tlib]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return out
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_py_extension())

@@ -1,66 +1,72 @@
-"""torch.nn.Module over the fused MoE launcher, shaped like the reference's
-vLLM wrapper (test/singleGPU/python/flashMoeOp.py:7-38): it takes the sparse
-MoE block of a Qwen3-MoE model, borrows `gate.weight`, `experts.w13_weight`
-and `experts.w2_weight`, runs the layer in place on `hidden_states`, and hands
-batches larger than `maxTokens` to the wrapped block.
+"""A sparse-MoE block that runs on the fused launcher.
 
-Differences from the reference wrapper: float32 and bfloat16 weights of any
-admitted shape (the reference: float32, the 30B shape only); `top_k` and an
-optional router bias are read from the block when it has them; a launch is a
-single kernel, so `forward` can be captured into a HIP graph; the fallback calls
-the wrapped block (the reference calls `super().forward`, which
-`torch.nn.Module` does not implement).
+`FlashMoeBlockWrapper(block, maxTokens)` stands in for the Qwen3-MoE block it is
+given, the way the reference's vLLM wrapper does
+(test/singleGPU/python/flashMoeOp.py:7-38): same class name, same first two
+constructor arguments, same attributes (`qwen3MoeSparseMoeBlockModule`,
+`launcher`, `maxTokens`), result written over `hidden_states`. The launcher is
+the compiled `flashMoeLauncher` extension; there is no fallback to Python code
+when it has not been built.
+
+What differs from the reference wrapper: float32 or bfloat16 weights of any
+admitted shape (the reference: float32, the 30B shape only); `top_k` and a router
+bias are taken from the block when it has them; a launch is one kernel, so
+`forward` can be captured into a HIP graph; batches beyond `maxTokens` go to the
+wrapped block itself (the reference calls `super().forward`, which
+`torch.nn.Module` does not define); the expert weights are packed once into the
+streaming layout unless `pack_weights=False`.
 """
+import os
+import sys
+
 import torch
 
-from . import flashMoeLauncher
+_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if _ROOT not in sys.path:
+    sys.path.insert(0, _ROOT)
+try:
+    import flashMoeLauncher
+except ImportError as e:  # no fallback: say how to build it
+    raise ImportError("the flashMoeLauncher extension is not built; run "
+                      "`python -m flash_distributed_moe_amd.build` (%s)" % e)
 
 
-def _block_top_k(block, default=8):
-    for owner in (block, getattr(block, "experts", None), getattr(block, "gate", None)):
-        for name in ("top_k", "num_experts_per_tok"):
-            v = getattr(owner, name, None)
+def _find_int(objs, names):
+    for o in objs:
+        for n in names:
+            v = getattr(o, n, None)
             if isinstance(v, int) and v > 0:
                 return v
-    return default
+    return None
 
 
 class FlashMoeBlockWrapper(torch.nn.Module):
 
     def __init__(self, qwen3MoeSparseMoeBlockModule, maxTokens, top_k=None, router_bias=None,
-                 pack_weights=False):
+                 pack_weights=True):
         super().__init__()
-        self.qwen3MoeSparseMoeBlockModule = qwen3MoeSparseMoeBlockModule
-        self.launcher = flashMoeLauncher.MoeKernelLauncher()
-
-        gateWeights = self.qwen3MoeSparseMoeBlockModule.gate.weight
-        ffn1ExpertWeights = self.qwen3MoeSparseMoeBlockModule.experts.w13_weight
-        ffn2ExpertWeights = self.qwen3MoeSparseMoeBlockModule.experts.w2_weight
+        block = qwen3MoeSparseMoeBlockModule
+        self.qwen3MoeSparseMoeBlockModule = block
+        self.maxTokens = int(maxTokens)
+        if top_k is None:
+            top_k = _find_int((block, getattr(block, "experts", None), getattr(block, "gate", None)),
+                              ("top_k", "num_experts_per_tok")) or 8
         if router_bias is None:
-            router_bias = getattr(self.qwen3MoeSparseMoeBlockModule.gate, "bias", None)
-
-        uniqueid = self.launcher.getDistributedUniqueId(empty=True)
+            router_bias = getattr(block.gate, "bias", None)
+        self.launcher = flashMoeLauncher.MoeKernelLauncher()
         self.launcher.create(
-            gateWeights, ffn1ExpertWeights, ffn2ExpertWeights, maxTokens, uniqueid, 0, 1,
-            top_k=top_k if top_k is not None else _block_top_k(qwen3MoeSparseMoeBlockModule),
-            router_bias=router_bias, pack_weights=pack_weights,
-        )
-        self.maxTokens = maxTokens
+            block.gate.weight, block.experts.w13_weight, block.experts.w2_weight, self.maxTokens,
+            self.launcher.getDistributedUniqueId(empty=True), 0, 1, top_k=int(top_k),
+            router_bias=router_bias,
+            flags=flashMoeLauncher.FLAG_PACK_WEIGHTS if pack_weights else 0)
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        if hidden_states.shape[0] > self.maxTokens:
+            return self.qwen3MoeSparseMoeBlockModule(hidden_states)
+        self.launcher.launch(hidden_states, hidden_states)  # output aliases input
+        return hidden_states
 
     def __del__(self):
         launcher = getattr(self, "launcher", None)
         if launcher is not None and launcher.valid:
             launcher.destroy()
-
-    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
-        num_tokens, _ = hidden_states.shape
-
-        if num_tokens <= self.maxTokens:
-            tokens = hidden_states
-
-            # Inplace calc -> output_mem = input_mem
-            self.launcher.launch(tokens, tokens)
-
-            return tokens
-        else:
-            return self.qwen3MoeSparseMoeBlockModule(hidden_states)

@@ -98,3 +98,17 @@ def test_python_launcher_surface():
         l.launch(None, None)
     l.destroy()                       # destroying an empty launcher is a no-op
     assert l.valid is False
+
+
+def test_drop_in_python_module_imports_by_the_reference_name():
+    """`import flashMoeLauncher` (test/singleGPU/python/flashMoeOp.py:1,
+    test_pythonBinding.py:2 of the reference) resolves to the compiled extension."""
+    import flashMoeLauncher
+
+    assert flashMoeLauncher.__file__.endswith(".so")
+    l = flashMoeLauncher.MoeKernelLauncher()
+    assert l.valid is False
+    uid = l.getDistributedUniqueId(empty=True)
+    assert isinstance(uid, bytes) and uid == bytes(128)
+    l.destroy()                       # a no-op on an empty launcher
+    assert l.valid is False

@@ -71,11 +71,15 @@ def test_wrapper_in_place_and_fallback(name, T):
     del layer
 
 
-def test_forward_in_hip_graph():
+@pytest.mark.parametrize("T", [32, 512])
+def test_forward_in_hip_graph(T):
     """A launch is one kernel and touches no host state, so it can be captured.
-    Every replay is checked against an eager launch on the same input, with
-    eager work and synchronisation between replays."""
-    cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=32)
+    Every replay gets fresh token contents and is checked bit for bit against an
+    eager launch of another launcher on the same input, with eager work and
+    synchronisation between replays. 32 tokens run the streaming variant, 512 the
+    tiled one (whose scratch rows are read with plain cached loads: a stale line
+    from the previous replay would show here)."""
+    cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=T)
     dev = torch.device("cuda:0")
     inp = synth.make_inputs_torch(cfg, 7907, dev)
     block = StandInSparseMoeBlock(inp, cfg.k)
@@ -106,3 +110,32 @@ def test_forward_in_hip_graph():
             ref = _oracle_out(cfg, inp, fresh)
             assert max_rel_err(work.float().cpu().numpy(), ref) <= 1e-2
     del layer, eager
+
+
+def test_python_binding_sequence_of_the_reference():
+    """The create / launch / destroy sequence of the reference's
+    test/singleGPU/python/test_pythonBinding.py:5-40, under the same import,
+    float32 at the reference's shape, plus what that test leaves out: the
+    result is checked against the oracle."""
+    import flashMoeLauncher
+
+    cfg = synth.MoeConfig("binding", 16, 2048, 128, 8, 768, "f32")
+    dev = torch.device("cuda:0")
+    inp = synth.make_inputs_torch(cfg, 123, dev)
+    tokens = inp["tokens"]
+    output = torch.empty_like(tokens)
+    launcher = flashMoeLauncher.MoeKernelLauncher()
+    assert launcher.valid == False  # noqa: E712
+    uniqueid = launcher.getDistributedUniqueId(empty=True)
+    launcher.create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T, uniqueid, 0, 1)
+    assert launcher.valid == True  # noqa: E712
+    launcher.launch(tokens, output)
+    torch.cuda.synchronize(dev)
+    assert output.shape == (cfg.T, cfg.H) and output.dtype == torch.float32
+    assert max_rel_err(output.cpu().numpy(), _oracle_out(cfg, inp, tokens)) <= 2e-5
+    with pytest.raises(RuntimeError, match="output shape"):
+        launcher.launch(tokens, output[:4])
+    launcher.destroy()
+    assert launcher.valid == False  # noqa: E712
+    with pytest.raises(RuntimeError, match="Launcher was destroyed"):
+        launcher.launch(tokens, output)
