@@ -64,7 +64,7 @@ class GpuCase:
         assert np.array_equal(routing["perm"], perm), "per-expert permutation differs"
         return idx, w
 
-    def check_outputs(self, tokens_t, out_t, token_ids=None):
+    def check_outputs(self, tokens_t, out_t, token_ids=None, nthreads=1):
         """Outputs of the chosen tokens (all when None) against the oracle."""
         hw = self.host_weights()
         x = tokens_t.float().cpu().numpy()
@@ -72,11 +72,13 @@ class GpuCase:
         if token_ids is not None:
             x, got = x[token_ids], got[token_ids]
         ref, _, _ = oracle.forward(x, hw["gate"], hw["ffn1"], hw["ffn2"], self.cfg.k,
-                                   bias=hw["bias"])
+                                   bias=hw["bias"], nthreads=nthreads)
         assert np.all(np.isfinite(got)), "non-finite output"
         err = max_rel_err(got, ref)
         tol = TOL[self.cfg.dtype]
         assert err <= tol, "max relative error %.3e > %.1e" % (err, tol)
         rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
-        np.testing.assert_allclose(got, ref, rtol=tol, atol=tol * rms * 4)
+        # elementwise as well: bf16 layers round every expert contribution of the tiled variant
+        # to bf16 before the slot sum, whose tail over 10^7 elements reaches 1.5 * tol * rms
+        np.testing.assert_allclose(got, ref, rtol=tol, atol=tol * rms * (2 if self.cfg.dtype == "bf16" else 1))
         return err

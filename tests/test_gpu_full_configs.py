@@ -1,8 +1,8 @@
-"""GPU parity at the full benchmark sizes. Routing is compared for every token
-(the oracle's router is cheap); outputs for a spread sample of tokens, since
-tokens are independent (a token's output depends only on its row and the
-weights). Size-independent properties cover the rest: permutation validity,
-determinism across launches, in-place == out-of-place."""
+"""GPU parity at the full benchmark sizes: routing and outputs of EVERY token
+against the oracle (its tokens dealt out over the host's cores: about 10 to 25 s
+per configuration on 16 cores), plus size-independent properties: permutation
+validity, determinism across launches, in-place == out-of-place."""
+import os
 import numpy as np
 import pytest
 import torch
@@ -27,7 +27,11 @@ def check_perm_properties(r, T, k, E):
     assert np.all(inner | boundary)                   # ascending (token, slot) inside a segment
 
 
-def run_full(name, sample, T=None, pack_weights=False):
+HOST_THREADS = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or 16))
+_first_output = {}   # (config, T) -> output of the first variant run: later variants must match it
+
+
+def run_full(name, T=None, pack_weights=False, same_bits_as_first=False):
     cfg = synth.CONFIGS[name]
     if T is not None:
         cfg = cfg.replace(T=T)
@@ -39,9 +43,16 @@ def run_full(name, sample, T=None, pack_weights=False):
         r = case.launcher.routing(cfg.T)
         case.check_routing(x, r)
         check_perm_properties(r, cfg.T, cfg.k, cfg.E)
-        ids = np.unique(np.linspace(0, cfg.T - 1, sample).astype(np.int64))
-        err = case.check_outputs(x, out, ids)
-        print("  max rel err %.3e on %d tokens" % (err, len(ids)), flush=True)
+        key = (cfg.name, cfg.T)
+        if same_bits_as_first and key in _first_output:
+            # same kernel, same operands: nothing may differ from the run already checked
+            assert torch.equal(out.cpu(), _first_output[key])
+            print("  bit-equal to the variant checked against the oracle", flush=True)
+        else:
+            err = case.check_outputs(x, out, None, nthreads=HOST_THREADS)
+            print("  max rel err %.3e on all %d tokens (%d host threads)" % (err, cfg.T, HOST_THREADS),
+                  flush=True)
+            _first_output[key] = out.cpu()
         out2 = case.run(inplace=True)
         assert torch.equal(out, out2)                 # deterministic; aliasing-safe
         return r
@@ -51,21 +62,22 @@ def run_full(name, sample, T=None, pack_weights=False):
 
 @pytest.mark.parametrize("pack_weights", [False, True])
 def test_qwen3_30b_prefill(pack_weights):
-    run_full("qwen3_30b_prefill", sample=48, pack_weights=pack_weights)
+    # the tiled variant reads the caller's layout either way
+    run_full("qwen3_30b_prefill", pack_weights=pack_weights, same_bits_as_first=True)
 
 
 @pytest.mark.parametrize("pack_weights", [False, True])
 def test_qwen3_235b_t256(pack_weights):
     # AUTO: the tiled variant on the caller's layout, the streaming one on the packed copy
-    run_full("qwen3_235b_t256", sample=24, pack_weights=pack_weights)
+    run_full("qwen3_235b_t256", pack_weights=pack_weights)
 
 
 def test_qwen3_235b_t4096():
-    run_full("qwen3_235b_t4096", sample=16)
+    run_full("qwen3_235b_t4096")
 
 
 def test_qwen3_30b_imbalance():
-    r = run_full("qwen3_30b_imbalance", sample=48)
+    r = run_full("qwen3_30b_imbalance")
     hot = synth.hot_experts(7907, 128, 4)
     share = r["counts"][hot].sum() / r["counts"].sum()
     print("  hot experts", hot, "share %.3f" % share, flush=True)
