@@ -52,6 +52,8 @@ C_ABI = {
     "flashMoeReadRouting": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
                                            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                            ctypes.c_void_p, ctypes.c_void_p]),
+    "flashMoeReadIntermediate": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
+                                                ctypes.c_void_p]),
     "flashMoeStatus": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint),
                                       ctypes.POINTER(ctypes.c_uint), ctypes.c_void_p]),
     "flashMoeSetWaitLimitMs": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_double]),

@@ -549,6 +549,18 @@ int flashMoeReadRouting(FlashMoeLauncher* l, int tokens_num, int* topk_idx, floa
   return hipSuccess;
 }
 
+int flashMoeReadIntermediate(FlashMoeLauncher* l, int tokens_num, void* h, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (l == nullptr || h == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null argument");
+  if (tokens_num < 0 || tokens_num > l->desc.max_tokens)
+    FMOE_FAIL(hipErrorInvalidValue, "tokens_num = %i", tokens_num);
+  FMOE_HIP_CHECK(hipStreamSynchronize(stream));
+  const size_t esz = l->desc.dtype == FLASH_MOE_BF16 ? 2 : 4;
+  const size_t bytes = esz * static_cast<size_t>(tokens_num) * l->desc.top_k * l->desc.intermediate;
+  FMOE_HIP_CHECK(hipMemcpy(h, l->ws + l->layout.h, bytes, hipMemcpyDeviceToHost));
+  return hipSuccess;
+}
+
 int flashMoeStatus(FlashMoeLauncher* l, unsigned* error_bits, unsigned* launches, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (l == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null launcher");

@@ -146,6 +146,19 @@ class MoeKernelLauncher:
         return dict(topk_idx=idx, topk_w=w, counts=counts, offsets=offsets,
                     perm=perm[:int(offsets[E])])
 
+    def intermediate(self, tokens_num):
+        """h of the last launch as float32 [tokens_num*k, I], rows in permuted order."""
+        if self._h is None:
+            raise RuntimeError("Launcher was destroyed")
+        _, _, inter, k = self._shape
+        raw = np.empty((tokens_num * k, inter), np.uint16 if self._dtype == torch.bfloat16 else np.float32)
+        with torch.cuda.device(self._device):
+            _hip_check(self._lib.flashMoeReadIntermediate(self._h, tokens_num, raw.ctypes.data, _stream()),
+                       "flashMoeReadIntermediate")
+        if raw.dtype == np.uint16:
+            return (raw.astype(np.uint32) << 16).view(np.float32)
+        return raw
+
     def status(self):
         """(error_bits, completed_launches) after waiting for the current stream."""
         err, n = ctypes.c_uint(), ctypes.c_uint()

@@ -124,6 +124,16 @@ int flashMoeDestroy(FlashMoeLauncher* l, void* stream);
 int flashMoeReadRouting(FlashMoeLauncher* l, int tokens_num, int* topk_idx, float* topk_w,
                         int* expert_counts, int* expert_offsets, int* perm, void* stream);
 
+/* After a launch of tokens_num tokens: waits for `stream`, then copies the
+ * expert stage's intermediate rows to the host: h [tokens_num*top_k, I] in the
+ * layer dtype, row r = SiLU(gate proj) * (up proj) of permuted row r (perm[r] of
+ * flashMoeReadRouting names its token and slot; rows from expert_offsets[E] on
+ * are unused). No counterpart in the reference's library; it is what lets a
+ * test compare the gate/up stage alone with the CPU reference, as the
+ * reference's stage test does
+ * (test/singleGPU/cpp/moe/internal/moeExpertFFN1Test.hip:58-106). */
+int flashMoeReadIntermediate(FlashMoeLauncher* l, int tokens_num, void* h, void* stream);
+
 /* Device-side failures. A dependency wait inside the kernel is bounded (see
  * flashMoeSetWaitLimitMs); when one runs out, or the row-tile table overflows,
  * the launch ends normally, its last worker fills the launch's output with NaN,
