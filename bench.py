@@ -34,16 +34,56 @@ BOUND = {
 }
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
-# dispatch) on exactly these workloads with the default seed and the packed weight copy; other
-# workloads have no measurement. Each counter is scaled by what it reads for a plain copy of
-# 1 GiB: WRITE_SIZE 1.000, FETCH_SIZE 0.500 (this chip reads HBM in 128-byte requests, which
-# the counter's formula prices at 64 bytes each).
+# HBM bytes per launch as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch)
+# live in profiles/traffic.json, one entry per workload, each with the digest of the kernel
+# sources it was measured on. An entry whose digest differs from the tree's is stale and is
+# not reported (traffic: null). `bench.py --record-traffic FETCH_KIB WRITE_KIB` writes the entry
+# of --config after a new pair of counter runs. Each counter is scaled by what it reads for a
+# plain copy of 1 GiB (bench.py --copy-calibration under the same counters): WRITE_SIZE 1.000,
+# FETCH_SIZE 0.500 (this chip reads HBM in 128-byte requests, which the counter's formula
+# prices at 64 bytes each).
 FETCH_SCALE = 0.5
-MEASURED_TRAFFIC = {
-    "qwen3_30b_decode": int(587847 / FETCH_SCALE + 6016) * 1024,
-    "qwen3_30b_prefill": int(1113843 / FETCH_SCALE + 429478) * 1024,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+KERNEL_SOURCES = ["moe_stream_kernel.hip", "moe_tiled_kernel.hip", "moe_device.h", "moe_params.h",
+                  "moe_launcher.hip"]
+
+
+def kernel_sources_digest():
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "flash_distributed_moe_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, packed):
+    """Bytes per launch from profiles/traffic.json, or None if there is no entry for this
+    workload and weight layout measured on the present kernel sources."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entry = json.load(f).get(workload)
+    except (OSError, ValueError):
+        return None
+    if not entry or entry.get("sources") != kernel_sources_digest() or \
+            bool(entry.get("packed_weight_copy")) != bool(packed):
+        return None
+    return int((entry["fetch_kib"] / entry["fetch_scale"] + entry["write_kib"]) * 1024)
+
+
+def record_traffic(workload, packed, fetch_kib, write_kib, kernel):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        table = {}
+    table[workload] = {"kernel": kernel, "fetch_kib": fetch_kib, "write_kib": write_kib,
+                       "fetch_scale": FETCH_SCALE, "packed_weight_copy": bool(packed),
+                       "sources": kernel_sources_digest()}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(table, f, indent=1, sort_keys=True)
+        f.write("\n")
 
 
 def algorithmic_bytes(cfg, active_experts):
@@ -98,68 +138,37 @@ def cpu_baseline(cfg, inp, seconds_budget=25.0):
     }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="qwen3_30b_decode")
-    ap.add_argument("--seed", type=int, default=7907)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sched", type=int, default=0)
-    ap.add_argument("--no-pack-weights", action="store_true",
-                    help="read the caller's weight layout instead of the packed second copy")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="only copy 1 GiB device to device five times: the known traffic the "
-                         "rocprofv3 byte counters are scaled by")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py: this build runs the MoE layer on ONE GPU (no collectives, no "
-                 "multi-GPU path); run with --gpus 1")
-
+def measure(name, seed, steps, warmup, sched, packed):
+    """K timed launches of workload `name`: whole-job wall time, the kernel's launch-to-launch
+    duration from events on the launch stream, and where that puts it on its roofline."""
     import torch
 
     from flash_distributed_moe_amd import synth
     from flash_distributed_moe_amd.flashMoeLauncher import MoeKernelLauncher
 
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible")
-    if args.copy_calibration:
-        a = torch.randn(1 << 28, device="cuda:0", dtype=torch.float32)
-        b = torch.empty_like(a)
-        for _ in range(5):
-            b.copy_(a)
-        torch.cuda.synchronize()
-        print(json.dumps({"copy_calibration": {"copies": 5, "kib_read_each": 1 << 20,
-                                               "kib_written_each": 1 << 20}}))
-        return
-    cfg = synth.CONFIGS[args.config]
+    cfg = synth.CONFIGS[name]
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    inp = synth.make_inputs_torch(cfg, args.seed, dev)
+    inp = synth.make_inputs_torch(cfg, seed, dev)
     x = inp["tokens"]
     out = torch.empty_like(x)
-
     launcher = MoeKernelLauncher()
     launcher.create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T,
                     launcher.getDistributedUniqueId(empty=True), 0, 1, top_k=cfg.k,
-                    router_bias=inp["bias"], sched=args.sched,
-                    pack_weights=not args.no_pack_weights)
-
-    for _ in range(args.warmup):
+                    router_bias=inp["bias"], sched=sched, pack_weights=packed)
+    for _ in range(warmup):
         launcher.launch(x, out)
     torch.cuda.synchronize()
 
     # whole-job wall time over exactly K steps
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         launcher.launch(x, out)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
+    ms_per_step = wall / steps * 1e3
 
     # per-launch kernel duration: events on the launch stream around single launches
-    n_ev = min(args.steps, 200)
+    n_ev = min(steps, 200)
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
            for _ in range(n_ev)]
     for a, b in evs:
@@ -176,33 +185,87 @@ def main():
         sys.exit("bench.py: device error bits %d" % err)
     routing = launcher.routing(cfg.T)
     active = int((routing["counts"] > 0).sum())
+    kernel = "moe_stream_kernel" if launcher.sched_for(cfg.T) == 1 else "moe_tiled_kernel"
+    launcher.destroy()
 
     bound = BOUND.get(cfg.name, "hbm")
     abytes = algorithmic_bytes(cfg, active)
     aflops = algorithmic_flops(cfg)
+    mfma_peak = MFMA_BF16_PEAK_TFLOPS if cfg.dtype == "bf16" else MFMA_F32_PEAK_TFLOPS
     if bound == "hbm":
         achieved = abytes / (kernel_ms_avg * 1e-3) / 1e9
         peak, unit = HBM_PEAK_GBS, "GB/s"
     else:
         achieved = aflops / (kernel_ms_avg * 1e-3) / 1e12
-        peak = MFMA_BF16_PEAK_TFLOPS if cfg.dtype == "bf16" else MFMA_F32_PEAK_TFLOPS
-        unit = "TFLOP/s"
+        peak, unit = mfma_peak, "TFLOP/s"
     roofline = {
         "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
         "frac": achieved / peak,
-        "traffic": MEASURED_TRAFFIC.get(cfg.name) if not args.no_pack_weights else None,
-        "kernel": "moe_stream_kernel" if launcher.sched_for(cfg.T) == 1 else "moe_tiled_kernel",
+        "traffic": measured_traffic(cfg.name, packed),
+        "kernel": kernel,
         "kernel_us_avg": kernel_ms_avg * 1e3, "kernel_us_median": kernel_ms_med * 1e3,
         "algorithmic_bytes": abytes, "algorithmic_flops": aflops, "active_experts": active,
         "hbm_frac": abytes / (kernel_ms_avg * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "mfma_frac": aflops / (kernel_ms_avg * 1e-3) / 1e12 /
-        (MFMA_BF16_PEAK_TFLOPS if cfg.dtype == "bf16" else MFMA_F32_PEAK_TFLOPS),
+        "mfma_frac": aflops / (kernel_ms_avg * 1e-3) / 1e12 / mfma_peak,
     }
+    config = {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E,
+              "top_k": cfg.k, "intermediate": cfg.I, "hot_experts": cfg.hot,
+              "seed": seed, "packed_weight_copy": packed}
+    return cfg, inp, ms_per_step, roofline, config
 
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="qwen3_30b_decode")
+    ap.add_argument("--seed", type=int, default=7907)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sched", type=int, default=0)
+    ap.add_argument("--no-pack-weights", action="store_true",
+                    help="read the caller's weight layout instead of the packed copy")
+    ap.add_argument("--no-extra-records", action="store_true",
+                    help="only the one workload: no prefill and no caller's-layout sub-record")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only copy 1 GiB device to device five times: the known traffic the "
+                         "rocprofv3 byte counters are scaled by")
+    ap.add_argument("--record-traffic", nargs=2, type=float, metavar=("FETCH_KIB", "WRITE_KIB"),
+                    help="no GPU work: write the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings "
+                         "(KiB per dispatch) of --config into profiles/traffic.json")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs the MoE layer on ONE GPU (no collectives, no "
+                 "multi-GPU path); run with --gpus 1")
+    packed = not args.no_pack_weights
+    if args.record_traffic:
+        kernel = "moe_tiled_kernel" if BOUND.get(args.config) == "mfma" or "4096" in args.config \
+            else "moe_stream_kernel"
+        record_traffic(args.config, packed, args.record_traffic[0], args.record_traffic[1], kernel)
+        print(json.dumps({args.config: measured_traffic(args.config, packed)}))
+        return
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    torch.cuda.set_device(0)
+    if args.copy_calibration:
+        a = torch.randn(1 << 28, device="cuda:0", dtype=torch.float32)
+        b = torch.empty_like(a)
+        for _ in range(5):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"copies": 5, "kib_read_each": 1 << 20,
+                                               "kib_written_each": 1 << 20}}))
+        return
+
+    cfg, inp, ms_per_step, roofline, config = measure(args.config, args.seed, args.steps,
+                                                      args.warmup, args.sched, packed)
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(cfg, inp)
-    launcher.destroy()
+    del inp
 
     line = {
         "metric": "MoE-layer tokens/s (Qwen3-style fused MoE forward, us/layer alongside)",
@@ -218,12 +281,23 @@ def main():
         "vs_baseline": None,
         "dtype": cfg.dtype,
         "data": "synthetic (seeded Irwin-Hall normal weights sigma 0.02, activations sigma 1)",
-        "config": {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E,
-                   "top_k": cfg.k, "intermediate": cfg.I, "hot_experts": cfg.hot,
-                   "seed": args.seed, "packed_weight_copy": not args.no_pack_weights},
+        "config": config,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
+    if not args.no_extra_records and args.config == "qwen3_30b_decode":
+        # the other headline workload (8192-token prefill, bound by the matrix cores) and the
+        # decode batch on the caller's weight layout (no packed copy), same fields
+        def sub(name, steps, warmup, packed_):
+            c, _, ms, roof, conf = measure(name, args.seed, steps, warmup, args.sched, packed_)
+            return {"value": c.T / (ms * 1e-3), "unit": "tokens/s", "steps": steps, "warmup": warmup,
+                    "ms_per_step": ms, "us_per_layer": ms * 1e3, "dtype": c.dtype, "config": conf,
+                    "roofline": roof}
+
+        line["prefill"] = sub("qwen3_30b_prefill", max(10, args.steps // 4), max(3, args.warmup // 4),
+                              packed)
+        if packed:
+            line["caller_layout"] = sub("qwen3_30b_decode", args.steps, args.warmup, False)
     print(json.dumps(line))
 
 
