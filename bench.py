@@ -67,7 +67,7 @@ def measured_traffic(workload, packed):
     except (OSError, ValueError):
         return None
     if not entry or entry.get("sources") != kernel_sources_digest() or \
-            bool(entry.get("packed_weight_copy")) != bool(packed):
+            bool(entry.get("packed_weights")) != bool(packed):
         return None
     return int((entry["fetch_kib"] / entry["fetch_scale"] + entry["write_kib"]) * 1024)
 
@@ -79,7 +79,7 @@ def record_traffic(workload, packed, fetch_kib, write_kib, kernel):
     except (OSError, ValueError):
         table = {}
     table[workload] = {"kernel": kernel, "fetch_kib": fetch_kib, "write_kib": write_kib,
-                       "fetch_scale": FETCH_SCALE, "packed_weight_copy": bool(packed),
+                       "fetch_scale": FETCH_SCALE, "packed_weights": bool(packed),
                        "sources": kernel_sources_digest()}
     with open(TRAFFIC_FILE, "w") as f:
         json.dump(table, f, indent=1, sort_keys=True)
@@ -152,9 +152,15 @@ def measure(name, seed, steps, warmup, sched, packed):
     x = inp["tokens"]
     out = torch.empty_like(x)
     launcher = MoeKernelLauncher()
-    launcher.create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T,
+    ffn1, ffn2 = inp["ffn1"], inp["ffn2"]
+    if packed:
+        # the layout the kernels read fastest, made where the tensors lie: the launcher keeps
+        # no copy of the weights (the row-major originals stay in `inp` for the CPU baseline)
+        ffn1, ffn2 = ffn1.clone(), ffn2.clone()
+        MoeKernelLauncher.pack_weights_in_place(ffn1, ffn2)
+    launcher.create(inp["gate"], ffn1, ffn2, cfg.T,
                     launcher.getDistributedUniqueId(empty=True), 0, 1, top_k=cfg.k,
-                    router_bias=inp["bias"], sched=sched, pack_weights=packed)
+                    router_bias=inp["bias"], sched=sched, prepacked=packed)
     for _ in range(warmup):
         launcher.launch(x, out)
     torch.cuda.synchronize()
@@ -210,7 +216,9 @@ def measure(name, seed, steps, warmup, sched, packed):
     }
     config = {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E,
               "top_k": cfg.k, "intermediate": cfg.I, "hot_experts": cfg.hot,
-              "seed": seed, "packed_weight_copy": packed}
+              "seed": seed, "packed_weight_copy": False,
+              "weights": "packed in place by the caller (flashMoePackWeightsInPlace), no second copy"
+                         if packed else "caller's row-major tensors"}
     return cfg, inp, ms_per_step, roofline, config
 
 
@@ -224,7 +232,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sched", type=int, default=0)
     ap.add_argument("--no-pack-weights", action="store_true",
-                    help="read the caller's weight layout instead of the packed copy")
+                    help="read the caller's row-major weight tensors instead of weights packed in place")
     ap.add_argument("--no-extra-records", action="store_true",
                     help="only the one workload: no prefill and no caller's-layout sub-record")
     ap.add_argument("--copy-calibration", action="store_true",

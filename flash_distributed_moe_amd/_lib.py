@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libflashMoe.so")
 F32, BF16 = 0, 1
 SCHED_AUTO, SCHED_STREAM, SCHED_TILED = 0, 1, 2
 FLAG_PACK_WEIGHTS = 1
+FLAG_WEIGHTS_PREPACKED = 2
 NOALLOC_SCRATCH_BYTES = 64 << 20
 HIP_SUCCESS = 0
 HIP_ERROR_INVALID_VALUE = 1
@@ -43,6 +44,8 @@ C_ABI = {
                                               ctypes.POINTER(ctypes.c_size_t)]),
     "flashMoeCreate": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(LayerDesc),
                                       ctypes.c_void_p]),
+    "flashMoePackWeights": (ctypes.c_int, [ctypes.c_int] * 5 + [ctypes.c_void_p] * 3),
+    "flashMoePackWeightsInPlace": (ctypes.c_int, [ctypes.c_int] * 5 + [ctypes.c_void_p] * 2),
     "flashMoeRefreshWeights": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p]),
     "flashMoeLaunch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                       ctypes.c_int, ctypes.c_void_p]),

@@ -135,8 +135,10 @@ hipError_t validate(const FlashMoeLayerDesc* d) {
               d->max_tokens, kMaxRows / d->top_k);
   if (d->sched < FLASH_MOE_SCHED_AUTO || d->sched > FLASH_MOE_SCHED_TILED)
     FMOE_FAIL(hipErrorInvalidValue, "sched = %i", d->sched);
-  if ((d->flags & ~FLASH_MOE_FLAG_PACK_WEIGHTS) != 0)
+  if ((d->flags & ~(FLASH_MOE_FLAG_PACK_WEIGHTS | FLASH_MOE_FLAG_WEIGHTS_PREPACKED)) != 0)
     FMOE_FAIL(hipErrorInvalidValue, "unknown flag bits 0x%x", d->flags);
+  if ((d->flags & FLASH_MOE_FLAG_PACK_WEIGHTS) && (d->flags & FLASH_MOE_FLAG_WEIGHTS_PREPACKED))
+    FMOE_FAIL(hipErrorInvalidValue, "weights that are already packed need no packed copy");
   return hipSuccess;
 }
 
@@ -158,7 +160,7 @@ int sched_for(const FlashMoeLayerDesc& d, int tokens_num) {
   if (!tiled_eligible(d, tokens_num)) return FLASH_MOE_SCHED_STREAM;
   if (d.sched == FLASH_MOE_SCHED_TILED) return FLASH_MOE_SCHED_TILED;
   const long long rows = static_cast<long long>(tokens_num) * d.top_k;
-  const bool packed = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
+  const bool packed = (d.flags & (FLASH_MOE_FLAG_PACK_WEIGHTS | FLASH_MOE_FLAG_WEIGHTS_PREPACKED)) != 0;
   return rows >= (packed ? 24ll : 3ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
 }
 
@@ -243,8 +245,10 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.ffn2 = d.ffn2_weights;
   p.bias = d.router_bias;
   const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
-  p.ffn1_packed = pack ? l->ws + L.pack1 : nullptr;
-  p.ffn2_packed = pack ? l->ws + L.pack2 : nullptr;
+  const bool prepacked = (d.flags & FLASH_MOE_FLAG_WEIGHTS_PREPACKED) != 0;
+  p.ffn1_packed = pack ? l->ws + L.pack1 : prepacked ? d.ffn1_weights : nullptr;
+  p.ffn2_packed = pack ? l->ws + L.pack2 : prepacked ? d.ffn2_weights : nullptr;
+  if (prepacked) p.ffn1 = p.ffn2 = nullptr;  // no row-major form exists
   p.out = output;
   char* w = l->ws;
   p.ctl = reinterpret_cast<fmoe::Control*>(w + L.ctl);
@@ -282,6 +286,51 @@ int flashMoeWorkspaceBytes(const FlashMoeLayerDesc* desc, size_t* bytes) {
   if (v != hipSuccess) return v;
   if (bytes == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null result pointer");
   *bytes = make_layout(*desc, may_run_tiled(*desc)).total;
+  return hipSuccess;
+}
+
+namespace {
+hipError_t check_pack_args(int dtype, int experts, int hidden, int intermediate, int which,
+                           const void* a, const void* b) {
+  if (dtype != FLASH_MOE_F32 && dtype != FLASH_MOE_BF16)
+    FMOE_FAIL(hipErrorInvalidValue, "dtype %i is neither float32 (0) nor bfloat16 (1)", dtype);
+  if (experts < 1 || hidden < 64 || hidden % 64 != 0 || intermediate < 32 || intermediate % 32 != 0)
+    FMOE_FAIL(hipErrorInvalidValue, "shape E=%i H=%i I=%i", experts, hidden, intermediate);
+  if (which != 0 && which != 1) FMOE_FAIL(hipErrorInvalidValue, "which = %i (0: ffn1, 1: ffn2)", which);
+  if (a == nullptr || b == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null weight pointer");
+  return hipSuccess;
+}
+}  // namespace
+
+int flashMoePackWeights(int dtype, int experts, int hidden, int intermediate, int which,
+                        const void* src, void* dst, void* stream_) {
+  const hipError_t v = check_pack_args(dtype, experts, hidden, intermediate, which, src, dst);
+  if (v != hipSuccess) return v;
+  if (src == dst) FMOE_FAIL(hipErrorInvalidValue, "src and dst must not overlap (see flashMoePackWeightsInPlace)");
+  FMOE_HIP_CHECK(fmoe::pack_weights(src, dst, dtype, experts, hidden, intermediate, which,
+                                    static_cast<hipStream_t>(stream_)));
+  return hipSuccess;
+}
+
+int flashMoePackWeightsInPlace(int dtype, int experts, int hidden, int intermediate, int which,
+                               void* weights, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const hipError_t v = check_pack_args(dtype, experts, hidden, intermediate, which, weights, weights);
+  if (v != hipSuccess) return v;
+  const size_t esz = dtype == FLASH_MOE_BF16 ? 2 : 4;
+  const size_t per_expert = esz * (which == 0 ? 2 : 1) * static_cast<size_t>(intermediate) * hidden;
+  void* staging = nullptr;
+  FMOE_HIP_CHECK(hipMalloc(&staging, per_expert));
+  hipError_t e = hipSuccess;
+  for (int x = 0; x < experts && e == hipSuccess; ++x) {
+    char* w = static_cast<char*>(weights) + per_expert * x;
+    e = hipMemcpyAsync(staging, w, per_expert, hipMemcpyDeviceToDevice, stream);
+    if (e == hipSuccess) e = fmoe::pack_weights(staging, w, dtype, 1, hidden, intermediate, which, stream);
+  }
+  const hipError_t s = hipStreamSynchronize(stream);
+  (void)hipFree(staging);
+  FMOE_HIP_CHECK(e);
+  FMOE_HIP_CHECK(s);
   return hipSuccess;
 }
 

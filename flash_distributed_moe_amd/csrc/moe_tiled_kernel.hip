@@ -487,8 +487,10 @@ constexpr int EPI_LD = TN * 2 + 16;              // bytes per row of the down ep
 static_assert(128 * EPI_LD <= TILE_LDS_BYTES, "epilogue slab exceeds the stage buffers");
 
 struct TileOperands {
-  const unsigned char* wbase;  // uniform: the weight matrix the offsets are relative to
+  const unsigned char* wbase;  // uniform: the weight matrix (or this wave's packed slice) the offsets are relative to
   const unsigned char* tbase;  // uniform: tokens, or h
+  unsigned wstride;            // uniform: bytes from one stage's weights to the next
+  bool wpacked;                // uniform: the weights come from the packed layout (see packed_run_offset)
   unsigned woff[NLD];          // this lane's 16 bytes of weight load q at stage 0
   unsigned toff[10];           // the same for the token rows
 };
@@ -548,7 +550,7 @@ __device__ __forceinline__ void tile_gemm(const TileOperands& op, int nstages, f
   auto issue_one = [&](int s, int q) {  // q: 0..7 weights, 8..8+NTL-1 tokens
     const unsigned st = uni(static_cast<int>(lds_addr + (s & 1) * STG));
     if (q < NLD) {
-      load_to_lds(op.woff[q], op.wbase + static_cast<size_t>(s) * ROWB, st + (wave * 64 + q * 8) * ROWB);
+      load_to_lds(op.woff[q], op.wbase + static_cast<size_t>(s) * op.wstride, st + (wave * 64 + q * 8) * ROWB);
     } else if (q < NLD + NTL) {
       const int qq = q - NLD;
       if ((NTL == 8 && JT == 8) || (wave * NTL + qq) * 8 < TROWS)
@@ -556,10 +558,20 @@ __device__ __forceinline__ void tile_gemm(const TileOperands& op, int nstages, f
                     st + TN * ROWB + ((wave * NTL + qq) * 8) * ROWB);
     }
   };
+  // weight fragments: from row-major stage rows as the token fragments, or, when the wave's
+  // weight rows keep the packed order (eight runs [k-step 0..1][block 0..3] of [chunk][row]),
+  // row r32 of 32-row block i = row r32 % 16 of run block 2i + r32 / 16, chunk 2*(u % 2) + kq
+  // of k-step u / 2
+  int ao[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    ao[u] = op.wpacked ? ((u >> 1) * 4 + (r32 >> 4)) * 1024 + (((2 * (u & 1) + kq) * 16 + (r32 & 15)) << 4)
+                       : fo[u];
+  const int ablock = uni(op.wpacked ? 2048 : 32 * ROWB);  // bytes from weight block 0 to block 1
   auto read_n = [&](Frag& f, int s, int u, int r) {  // r-th of the NRD reads of a sub-step
     const unsigned char* st = lds_raw + (s & 1) * STG + fo[u];
     if (r < 2) {
-      f.a[r] = *reinterpret_cast<const uint4*>(st + (wave * 64 + r * 32) * ROWB);
+      f.a[r] = *reinterpret_cast<const uint4*>(lds_raw + (s & 1) * STG + wave * (64 * ROWB) + r * ablock + ao[u]);
     } else if (r < NRD) {
       f.b[r - 2] = *reinterpret_cast<const uint4*>(st + TN * ROWB + ((r - 2) * 32) * ROWB);
     }
@@ -677,6 +689,20 @@ __device__ __forceinline__ void tile_gemm(const TileOperands& op, int nstages, f
   __syncthreads();  // the stages are free for the epilogue
 }
 
+// Weights in the packed layout (the streaming variant's: per wave task and 32-k step four
+// runs of 1 KiB, one per 16-row block, each [16-byte chunk 0..3][row 0..15]). This wave's 64
+// stage rows are exactly one packed task: gate/up task (expert, 32 h columns) = gate blocks
+// 0,1 and up blocks 2,3; down task (expert, 64 output columns) = blocks 0..3. A stage of 64 k
+// is two 32-k steps, i.e. eight runs, and load q of the wave copies run (k-step q / 4, block
+// q % 4) as it is: eight whole lines read by consecutive lanes. (Permuting the chunks into the
+// row-major stage layout on the way in made every 16 lanes touch 8 lines: prefill 798 -> 867 us.)
+// So with packed weights the wave's weight rows keep the packed order in LDS, and only the
+// fragment reads differ: see tile_gemm.
+static_assert(G1_NB == 2 && G2_NB == 4, "the tiled variant reads the packed layout as 32+32-row and 64-row tasks");
+__device__ __forceinline__ unsigned packed_run_offset(int q) {
+  return static_cast<unsigned>((q >> 2) * 4096 + (q & 3) * 1024 + (threadIdx.x & 63) * 16);
+}
+
 // One GEMM tile task, gate/up or down, for a row tile of up to 32*JT rows.
 //
 // gate/up: h[row, n0 .. n0+128) (test/singleGPU/cpp/moe/reference/refExpertFFN1.h:51-65).
@@ -705,7 +731,17 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
   int nstages;
   if (down) {
     nstages = I / KS;
-    op.wbase = uni(reinterpret_cast<const unsigned char*>(p.ffn2)) + (static_cast<size_t>(expert) * H + n0) * I * 2;
+    const bool packed = uni(p.ffn2_packed != nullptr ? 1 : 0) != 0;
+    if (packed) {
+      const size_t task = static_cast<size_t>(expert) * (H / 64) + (n0 / 64 + wave);
+      op.wbase = uni(reinterpret_cast<const unsigned char*>(p.ffn2_packed)) + task * (static_cast<size_t>(I / 32) * 4096);
+      op.wstride = 8192u;
+      op.wpacked = true;
+    } else {
+      op.wpacked = false;
+      op.wbase = uni(reinterpret_cast<const unsigned char*>(p.ffn2)) + (static_cast<size_t>(expert) * H + n0) * I * 2;
+      op.wstride = static_cast<unsigned>(ROWB);
+    }
     op.tbase = uni(reinterpret_cast<const unsigned char*>(p.h)) + static_cast<size_t>(row0) * I * 2;
     const float* row_w = uni(p.row_w) + row0;
 #pragma unroll
@@ -717,7 +753,8 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
 #pragma unroll
     for (int q = 0; q < NLD; ++q) {
       const int row = stage_row(NLD, q);
-      op.woff[q] = static_cast<unsigned>(row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
+      op.woff[q] = packed ? packed_run_offset(q)
+                          : static_cast<unsigned>(row) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
     }
 #pragma unroll
     for (int q = 0; q < NTL; ++q) {
@@ -726,7 +763,17 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
     }
   } else {
     nstages = H / KS;
-    op.wbase = uni(reinterpret_cast<const unsigned char*>(p.ffn1)) + static_cast<size_t>(expert) * 2 * I * H * 2;
+    const bool packed = uni(p.ffn1_packed != nullptr ? 1 : 0) != 0;
+    if (packed) {
+      const size_t task = static_cast<size_t>(expert) * (I / 32) + (n0 / 32 + wave);
+      op.wbase = uni(reinterpret_cast<const unsigned char*>(p.ffn1_packed)) + task * (static_cast<size_t>(H / 32) * 4096);
+      op.wstride = 8192u;
+      op.wpacked = true;
+    } else {
+      op.wpacked = false;
+      op.wbase = uni(reinterpret_cast<const unsigned char*>(p.ffn1)) + static_cast<size_t>(expert) * 2 * I * H * 2;
+      op.wstride = static_cast<unsigned>(ROWB);
+    }
     op.tbase = uni(reinterpret_cast<const unsigned char*>(p.tokens));
 #pragma unroll
     for (int q = 0; q < NLD; ++q) {
@@ -734,7 +781,8 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
       // weight stage rows 64w..64w+31: gate rows n0+32w.., 64w+32..64w+63: up rows I+n0+32w..
       const int wl = row & 63;
       const int wrow = (wl < 32 ? n0 : I + n0 - 32) + 32 * wave + wl;
-      op.woff[q] = static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
+      op.woff[q] = packed ? packed_run_offset(q)
+                          : static_cast<unsigned>(wrow) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
     }
 #pragma unroll
     for (int q = 0; q < NTL; ++q) {

@@ -138,6 +138,27 @@ class Launcher {
   int64_t hidden_ = 0;
 };
 
+// Rewrites ffn1 [E,2I,H] and ffn2 [E,H,I] into the packed layout where they lie (no second
+// copy); create(..., flags=FLAG_WEIGHTS_PREPACKED) takes them afterwards.
+void pack_weights_in_place(const at::Tensor& ffn1, const at::Tensor& ffn2) {
+  check_tensor(ffn1, "ffn1_expert_weights");
+  check_tensor(ffn2, "ffn2_expert_weights");
+  TORCH_CHECK(ffn1.dim() == 3 && ffn2.dim() == 3 && ffn1.scalar_type() == ffn2.scalar_type(),
+              "weights must be [E,2I,H] and [E,H,I] of one dtype");
+  const int experts = static_cast<int>(ffn1.size(0)), hidden = static_cast<int>(ffn1.size(2)),
+            inter = static_cast<int>(ffn2.size(2));
+  TORCH_CHECK(ffn1.size(1) == 2 * inter && ffn2.size(0) == experts && ffn2.size(1) == hidden,
+              "weights must be [E,2I,H] and [E,H,I]");
+  const int dtype = ffn1.scalar_type() == at::kBFloat16 ? FLASH_MOE_BF16 : FLASH_MOE_F32;
+  const DeviceGuard guard(ffn1.device());
+  check_hip(static_cast<hipError_t>(flashMoePackWeightsInPlace(dtype, experts, hidden, inter, 0,
+                                                               ffn1.data_ptr(), current_stream())),
+            "flashMoePackWeightsInPlace");
+  check_hip(static_cast<hipError_t>(flashMoePackWeightsInPlace(dtype, experts, hidden, inter, 1,
+                                                               ffn2.data_ptr(), current_stream())),
+            "flashMoePackWeightsInPlace");
+}
+
 }  // namespace
 
 PYBIND11_MODULE(flashMoeLauncher, m) {
@@ -146,6 +167,9 @@ PYBIND11_MODULE(flashMoeLauncher, m) {
   m.attr("SCHED_STREAM") = static_cast<int>(FLASH_MOE_SCHED_STREAM);
   m.attr("SCHED_TILED") = static_cast<int>(FLASH_MOE_SCHED_TILED);
   m.attr("FLAG_PACK_WEIGHTS") = static_cast<int>(FLASH_MOE_FLAG_PACK_WEIGHTS);
+  m.attr("FLAG_WEIGHTS_PREPACKED") = static_cast<int>(FLASH_MOE_FLAG_WEIGHTS_PREPACKED);
+  m.def("pack_weights_in_place", &pack_weights_in_place, py::arg("ffn1_expert_weights"),
+        py::arg("ffn2_expert_weights"));
   py::class_<Launcher>(m, "MoeKernelLauncher")
       .def(py::init())
       .def_static("getDistributedUniqueId", &Launcher::unique_id, py::arg("empty") = false,

@@ -61,7 +61,7 @@ class MoeKernelLauncher:
 
     def create(self, gate_weights, ffn1_expert_weights, ffn2_expert_weights, max_tokens, uid,
                rank, world_size, top_k=8, router_bias=None, sched=_lib.SCHED_AUTO,
-               pack_weights=False):
+               pack_weights=False, prepacked=False):
         _check(self._h is None, "Launcher already created")
         for t, n in ((gate_weights, "gate_weights"), (ffn1_expert_weights, "ffn1_expert_weights"),
                      (ffn2_expert_weights, "ffn2_expert_weights")):
@@ -93,7 +93,9 @@ class MoeKernelLauncher:
         d.experts, d.hidden, d.intermediate, d.top_k = experts, hidden, inter, int(top_k)
         d.dtype = _lib.BF16 if gate_weights.dtype == torch.bfloat16 else _lib.F32
         d.max_tokens, d.sched = int(max_tokens), int(sched)
-        d.flags = _lib.FLAG_PACK_WEIGHTS if pack_weights else 0
+        _check(not (pack_weights and prepacked), "prepacked weights need no packed copy")
+        d.flags = (_lib.FLAG_PACK_WEIGHTS if pack_weights else 0) | \
+                  (_lib.FLAG_WEIGHTS_PREPACKED if prepacked else 0)
         d.gate_weights = gate_weights.data_ptr()
         d.ffn1_weights = ffn1_expert_weights.data_ptr()
         d.ffn2_weights = ffn2_expert_weights.data_ptr()
@@ -108,6 +110,24 @@ class MoeKernelLauncher:
         # weights are borrowed by the library: keep them alive with the launcher
         self._keep = (gate_weights, ffn1_expert_weights, ffn2_expert_weights, router_bias)
         self._device = gate_weights.device
+
+    @staticmethod
+    def pack_weights_in_place(ffn1_expert_weights, ffn2_expert_weights):
+        """Rewrites the two expert tensors ([E,2I,H], [E,H,I]) into the packed layout where
+        they lie (no second copy); pass them to create(..., prepacked=True) afterwards.
+        Their contents are no longer row-major matrices after this."""
+        lib = _lib.load()
+        _check_tensor(ffn1_expert_weights, "ffn1_expert_weights")
+        _check_tensor(ffn2_expert_weights, "ffn2_expert_weights")
+        experts, two_i, hidden = ffn1_expert_weights.shape
+        inter = two_i // 2
+        _check(tuple(ffn2_expert_weights.shape) == (experts, hidden, inter), "ffn2 must be [E,H,I]")
+        dt = _lib.BF16 if ffn1_expert_weights.dtype == torch.bfloat16 else _lib.F32
+        with torch.cuda.device(ffn1_expert_weights.device):
+            for which, t in ((0, ffn1_expert_weights), (1, ffn2_expert_weights)):
+                _hip_check(lib.flashMoePackWeightsInPlace(dt, experts, hidden, inter, which,
+                                                          t.data_ptr(), _stream()),
+                           "flashMoePackWeightsInPlace")
 
     def launch(self, tokens, output):
         if self._h is None:

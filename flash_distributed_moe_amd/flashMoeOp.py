@@ -13,8 +13,12 @@ admitted shape (the reference: float32, the 30B shape only); `top_k` and a route
 bias are taken from the block when it has them; a launch is one kernel, so
 `forward` can be captured into a HIP graph; batches beyond `maxTokens` go to the
 wrapped block itself (the reference calls `super().forward`, which
-`torch.nn.Module` does not define); the expert weights are packed once into the
-streaming layout unless `pack_weights=False`.
+`torch.nn.Module` does not define). `pack_weights` says how the kernels get the
+packed weight layout they read fastest: True (default) keeps a packed second
+copy inside the launcher and leaves the block's tensors alone; "in_place"
+rewrites the block's `w13_weight` / `w2_weight` into the packed layout where they
+lie (no extra memory; the wrapped block can then no longer compute with them, so
+`maxTokens` must cover every batch); False reads the row-major tensors.
 """
 import os
 import sys
@@ -53,15 +57,23 @@ class FlashMoeBlockWrapper(torch.nn.Module):
                               ("top_k", "num_experts_per_tok")) or 8
         if router_bias is None:
             router_bias = getattr(block.gate, "bias", None)
+        self.weights_in_place = pack_weights == "in_place"
+        if self.weights_in_place:
+            flashMoeLauncher.pack_weights_in_place(block.experts.w13_weight.data, block.experts.w2_weight.data)
+            flags = flashMoeLauncher.FLAG_WEIGHTS_PREPACKED
+        else:
+            flags = flashMoeLauncher.FLAG_PACK_WEIGHTS if pack_weights else 0
         self.launcher = flashMoeLauncher.MoeKernelLauncher()
         self.launcher.create(
             block.gate.weight, block.experts.w13_weight, block.experts.w2_weight, self.maxTokens,
             self.launcher.getDistributedUniqueId(empty=True), 0, 1, top_k=int(top_k),
-            router_bias=router_bias,
-            flags=flashMoeLauncher.FLAG_PACK_WEIGHTS if pack_weights else 0)
+            router_bias=router_bias, flags=flags)
 
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
         if hidden_states.shape[0] > self.maxTokens:
+            if self.weights_in_place:
+                raise RuntimeError("batch of %d tokens exceeds maxTokens = %d and the wrapped block's "
+                                   "weights were packed in place" % (hidden_states.shape[0], self.maxTokens))
             return self.qwen3MoeSparseMoeBlockModule(hidden_states)
         self.launcher.launch(hidden_states, hidden_states)  # output aliases input
         return hidden_states

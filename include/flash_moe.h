@@ -42,13 +42,21 @@ enum { FLASH_MOE_F32 = 0, FLASH_MOE_BF16 = 1 };
 /* Scheduling variant. AUTO picks by rows per expert. */
 enum { FLASH_MOE_SCHED_AUTO = 0, FLASH_MOE_SCHED_STREAM = 1, FLASH_MOE_SCHED_TILED = 2 };
 
-/* FLASH_MOE_FLAG_PACK_WEIGHTS: at create the expert weights are copied once into
- * a layout of contiguous 1 KiB runs (16 rows x 32 k) that the streaming
- * (small-batch) variant reads front to back and the tiled variant loads as
- * whole cache lines; costs a second copy of the expert weights in device
- * memory. The caller's tensors stay the external format and are no longer read
- * by launches; after changing them call flashMoeRefreshWeights. */
-enum { FLASH_MOE_FLAG_PACK_WEIGHTS = 1 };
+/* The packed weight layout: contiguous 1 KiB runs (16 rows x 32 k) in the order
+ * the kernels' tasks read them, which the streaming (small-batch) variant reads
+ * front to back and the tiled variant loads as whole cache lines; same size as
+ * the row-major tensors. Three ways to use it:
+ *  FLASH_MOE_FLAG_PACK_WEIGHTS      at create the library copies the caller's
+ *      row-major expert weights into a packed second copy in its workspace
+ *      (+3*E*H*I elements of device memory). The caller's tensors stay the external
+ *      format and are no longer read by launches; after changing them call
+ *      flashMoeRefreshWeights.
+ *  FLASH_MOE_FLAG_WEIGHTS_PREPACKED ffn1_weights / ffn2_weights already hold the
+ *      packed layout (made by flashMoePackWeights into buffers of the caller's, or
+ *      by flashMoePackWeightsInPlace): no second copy anywhere; the row-major form
+ *      need not exist any more.
+ *  neither                          launches read the caller's row-major tensors. */
+enum { FLASH_MOE_FLAG_PACK_WEIGHTS = 1, FLASH_MOE_FLAG_WEIGHTS_PREPACKED = 2 };
 
 typedef struct FlashMoeLayerDesc {
   int experts;      /* E, 1..256 */
@@ -73,6 +81,19 @@ int flashMoeWorkspaceBytes(const FlashMoeLayerDesc* desc, size_t* bytes);
  * untouched. hipErrorUnknown: max_tokens beyond capacity;
  * hipErrorInvalidValue: anything else wrong with the description. */
 int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* stream);
+
+/* Packs expert weights for FLASH_MOE_FLAG_WEIGHTS_PREPACKED. which = 0: src is
+ * ffn1 [experts, 2I, H]; which = 1: src is ffn2 [experts, H, I]; row-major,
+ * dtype FLASH_MOE_F32 or FLASH_MOE_BF16, device memory. flashMoePackWeights writes
+ * the packed form to dst (same size, must not overlap src), enqueued on `stream`.
+ * flashMoePackWeightsInPlace rewrites the tensor where it lies, one expert at a
+ * time through a staging buffer of one expert's matrix that it allocates and
+ * frees; it waits for `stream`. No counterpart in the reference, which reads the
+ * caller's layout only (src/hip/launcher/moeKernelLauncher.hip:107-109). */
+int flashMoePackWeights(int dtype, int experts, int hidden, int intermediate, int which,
+                        const void* src, void* dst, void* stream);
+int flashMoePackWeightsInPlace(int dtype, int experts, int hidden, int intermediate, int which,
+                               void* weights, void* stream);
 
 /* Re-reads the caller's expert weights into the packed copy (no-op without
  * FLASH_MOE_FLAG_PACK_WEIGHTS). Enqueued on `stream`. No counterpart in the

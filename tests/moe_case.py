@@ -16,7 +16,7 @@ TOL = {"bf16": 1e-2, "f32": 2e-5}
 
 class GpuCase:
     def __init__(self, cfg, seed=7907, sched=_lib.SCHED_AUTO, max_tokens=None, inputs=None,
-                 pack_weights=False):
+                 pack_weights=False, prepacked=False):
         self.cfg, self.seed = cfg, seed
         self.dev = torch.device("cuda:0")
         self.inp = inputs or synth.make_inputs_torch(cfg, seed, self.dev)
@@ -25,7 +25,7 @@ class GpuCase:
         self.launcher.create(self.inp["gate"], self.inp["ffn1"], self.inp["ffn2"],
                              max_tokens or cfg.T, uid, 0, 1, top_k=cfg.k,
                              router_bias=self.inp["bias"], sched=sched,
-                             pack_weights=pack_weights)
+                             pack_weights=pack_weights, prepacked=prepacked)
 
     def run(self, tokens=None, inplace=False):
         x = self.inp["tokens"] if tokens is None else tokens

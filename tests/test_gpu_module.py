@@ -139,3 +139,24 @@ def test_python_binding_sequence_of_the_reference():
     assert launcher.valid == False  # noqa: E712
     with pytest.raises(RuntimeError, match="Launcher was destroyed"):
         launcher.launch(tokens, output)
+
+
+def test_wrapper_packs_the_blocks_weights_in_place():
+    """pack_weights="in_place": the block's expert tensors are rewritten into the
+    packed layout (no second copy); results as with the row-major tensors, and a
+    batch beyond maxTokens is an error instead of a wrong answer from the wrapped block."""
+    cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=24)
+    dev = torch.device("cuda:0")
+    inp = synth.make_inputs_torch(cfg, 7907, dev)
+    mine = dict(inp, ffn1=inp["ffn1"].clone(), ffn2=inp["ffn2"].clone())
+    layer = FlashMoeBlockWrapper(StandInSparseMoeBlock(mine, cfg.k), maxTokens=cfg.T, pack_weights="in_place")
+    assert not torch.equal(mine["ffn1"], inp["ffn1"])
+    plain = FlashMoeBlockWrapper(StandInSparseMoeBlock(inp, cfg.k), maxTokens=cfg.T, pack_weights=False)
+    x = inp["tokens"]
+    got, want = layer(x.clone()), plain(x.clone())
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert max_rel_err(got.float().cpu().numpy(), _oracle_out(cfg, inp, x)) <= 1e-2
+    with pytest.raises(RuntimeError, match="packed in place"):
+        layer(torch.cat([x, x], 0))
+    del layer, plain

@@ -220,3 +220,48 @@ def test_packed_weights_equal_unpacked(name, T):
             b.close()
     finally:
         a.close()
+
+
+@pytest.mark.parametrize("name,T,sched", [("qwen3_30b_decode", 64, _lib.SCHED_STREAM),
+                                          ("qwen3_30b_decode", 700, _lib.SCHED_TILED),
+                                          ("tiny_f32", 16, _lib.SCHED_STREAM)])
+def test_prepacked_weights_equal_unpacked(name, T, sched):
+    """Weights packed in place by the caller (no second copy anywhere, the
+    launcher's workspace holds no weight-sized region) give the same bits as the
+    row-major tensors and as the launcher's own packed copy."""
+    import ctypes
+
+    cfg = synth.CONFIGS[name].replace(T=T)
+    a = GpuCase(cfg, seed=11, sched=sched)
+    try:
+        out_a = a.run()
+        packed_inp = dict(a.inp)
+        packed_inp["ffn1"] = a.inp["ffn1"].clone()
+        packed_inp["ffn2"] = a.inp["ffn2"].clone()
+        a.launcher.pack_weights_in_place(packed_inp["ffn1"], packed_inp["ffn2"])
+        torch.cuda.synchronize()
+        assert not torch.equal(packed_inp["ffn1"], a.inp["ffn1"])     # it really is another layout
+        b = GpuCase(cfg, seed=11, sched=sched, inputs=packed_inp, prepacked=True)
+        try:
+            assert torch.equal(b.run(), out_a)
+            b.check_routing(b.inp["tokens"], b.launcher.routing(T))
+            # workspace: nothing weight-sized
+            d = _lib.LayerDesc()
+            d.experts, d.hidden, d.intermediate, d.top_k = cfg.E, cfg.H, cfg.I, cfg.k
+            d.dtype = _lib.BF16 if cfg.dtype == "bf16" else _lib.F32
+            d.max_tokens, d.sched, d.flags = T, sched, _lib.FLAG_WEIGHTS_PREPACKED
+            n_pre, n_copy = ctypes.c_size_t(0), ctypes.c_size_t(0)
+            assert _lib.load().flashMoeWorkspaceBytes(ctypes.byref(d), ctypes.byref(n_pre)) == 0
+            d.flags = _lib.FLAG_PACK_WEIGHTS
+            assert _lib.load().flashMoeWorkspaceBytes(ctypes.byref(d), ctypes.byref(n_copy)) == 0
+            esz = 2 if cfg.dtype == "bf16" else 4
+            assert n_copy.value - n_pre.value >= 3 * cfg.E * cfg.H * cfg.I * esz
+        finally:
+            b.close()
+        c = GpuCase(cfg, seed=11, sched=sched, inputs=a.inp, pack_weights=True)
+        try:
+            assert torch.equal(c.run(), out_a)
+        finally:
+            c.close()
+    finally:
+        a.close()
