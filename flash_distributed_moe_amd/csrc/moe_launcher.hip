@@ -31,6 +31,7 @@ hipError_t prepare_tiled_kernel();
 hipError_t stream_kernel_occupancy(int dtype, int* per_cu);
 hipError_t tiled_kernel_occupancy(int* per_cu);
 int tiled_max_tokens();
+size_t tiled_y_bytes(size_t rows, size_t hidden);
 }
 
 #define FMOE_FILENAME (strrchr(__FILE__, '/') ? strrchr(__FILE__, '/') + 1 : __FILE__)
@@ -102,7 +103,16 @@ Layout make_layout(const FlashMoeLayerDesc& d, bool need_tiled) {
   (void)need_tiled;  // both variants keep h as [rows, I], rows in permuted order
   const size_t h_rows = rows;
   L.h = take(esz * h_rows * d.intermediate);
-  L.y = take(sizeof(float) * rows * d.hidden);
+  // y: the streaming variant keeps every (token, slot) row in float, the tiled variant in
+  // bf16. When every batch that asks for the tiled variant gets it (tiled_all) and AUTO hands
+  // it the large batches, the streaming one only ever sees batches below the switch-over.
+  const bool tiled_all = need_tiled && static_cast<long long>(d.max_tokens) * d.hidden * 2 < (1ll << 32);
+  const size_t stream_rows =
+      tiled_all && d.sched == FLASH_MOE_SCHED_TILED ? 0
+      : tiled_all && d.sched == FLASH_MOE_SCHED_AUTO ? std::min<size_t>(rows, 24 * static_cast<size_t>(d.experts))
+                                                     : rows;
+  L.y = take(std::max(sizeof(float) * stream_rows * d.hidden,
+                      need_tiled ? fmoe::tiled_y_bytes(rows, d.hidden) : 0));
   const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
   L.pack1 = take(pack ? esz * d.experts * 2 * d.intermediate * d.hidden : 0);
   L.pack2 = take(pack ? esz * d.experts * d.hidden * d.intermediate : 0);

@@ -944,34 +944,52 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
   unsigned char* flag = lds_raw;  // [CMB_TOK * MAX_TOPK]
   if (tid < ntok * K) flag[tid] = ldc(&topk_idx[static_cast<size_t>(t0) * K + tid]) >= 0 ? 1 : 0;
   __syncthreads();
-  // one item = 8 columns of one token; the K row loads of an item are in flight together
+  // one item = 8 columns of one token; a thread works on two items at a time, so that 2*K
+  // row loads are in flight per lane (one CU alone needs about 64 KiB in flight for its share
+  // of the memory bandwidth)
   const int cpr = H >> 3;  // items per token
-  for (int it = tid; it < ntok * cpr; it += T_THREADS) {
-    const int tl = it / cpr, c = (it - tl * cpr) << 3;
-    const int t = t0 + tl;
-    unsigned valid = 0u;
-    for (int k = 0; k < K; ++k) valid |= static_cast<unsigned>(flag[tl * K + k]) << k;
-    const unsigned short* yrow = y + static_cast<size_t>(t) * K * H + c;
-    float s[8];
+  const int nitems = ntok * cpr;
+  for (int it0 = tid; it0 < nitems; it0 += 2 * T_THREADS) {
+    float s[2][8];
+    unsigned valid[2];
+    const unsigned short* yrow[2];
+    int tok[2], col[2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) s[i] = 0.0f;
-    for (int k0 = 0; k0 < K; k0 += 8) {
-      uint4 v[8];
+    for (int u = 0; u < 2; ++u) {
+      const int it = min(it0 + u * T_THREADS, nitems - 1);
+      const int tl = it / cpr;
+      col[u] = (it - tl * cpr) << 3;
+      tok[u] = t0 + tl;
+      valid[u] = 0u;
+      for (int k = 0; k < K; ++k) valid[u] |= static_cast<unsigned>(flag[tl * K + k]) << k;
+      yrow[u] = y + static_cast<size_t>(tok[u]) * K * H + col[u];
 #pragma unroll
-      for (int k = 0; k < 8; ++k)
-        if (k0 + k < K) v[k] = ld16_once(yrow + static_cast<size_t>(k0 + k) * H);
-#pragma unroll
-      for (int k = 0; k < 8; ++k)
-        if (k0 + k < K && ((valid >> (k0 + k)) & 1u)) {
-          float f[8];
-          unpack<BF16>(v[k], f);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) s[i] += f[i];
-        }
+      for (int i = 0; i < 8; ++i) s[u][i] = 0.0f;
     }
-    st16(out + static_cast<size_t>(t) * H + c,
-         u32x4{pack_bf16(s[0], s[1]), pack_bf16(s[2], s[3]), pack_bf16(s[4], s[5]),
-               pack_bf16(s[6], s[7])});
+    for (int k0 = 0; k0 < K; k0 += 8) {
+      uint4 v[2][8];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (k0 + k < K) v[u][k] = ld16_once(yrow[u] + static_cast<size_t>(k0 + k) * H);
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (k0 + k < K && ((valid[u] >> (k0 + k)) & 1u)) {
+            float f[8];
+            unpack<BF16>(v[u][k], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s[u][i] += f[i];
+          }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      if (it0 + u * T_THREADS < nitems)
+        st16(out + static_cast<size_t>(tok[u]) * H + col[u],
+             u32x4{pack_bf16(s[u][0], s[u][1]), pack_bf16(s[u][2], s[u][3]), pack_bf16(s[u][4], s[u][5]),
+                   pack_bf16(s[u][6], s[u][7])});
   }
   for (int tl = 0; tl < ntok; ++tl) {
     const int t = t0 + tl;
@@ -1214,6 +1232,8 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
 
 // Largest token count of the tiled variant: the launcher's capacity at top-1.
 int tiled_max_tokens() { return 1 << 21; }
+// y of the tiled variant: one bf16 row of H per (token, slot)
+size_t tiled_y_bytes(size_t rows, size_t hidden) { return rows * hidden * 2; }
 
 hipError_t launch_tiled_kernel(const Params& p, int grid, hipStream_t stream) {
   hipLaunchKernelGGL(moe_tiled_kernel, dim3(grid), dim3(T_THREADS), TILED_LDS_BYTES, stream, p);

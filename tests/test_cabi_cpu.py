@@ -54,8 +54,12 @@ def test_workspace_size_grows_with_tokens():
     rc1, n1 = workspace(desc(max_tokens=64))
     rc2, n2 = workspace(desc(max_tokens=8192))
     assert rc1 == 0 and rc2 == 0 and n2 > n1 > 0
-    # y [T*k, H] float + h [T*k, I] bf16 dominate
-    assert n2 >= 8192 * 8 * (2048 * 4 + 768 * 2)
+    rows = 8192 * 8
+    # at prefill sizes h [T*k, I] and y [T*k, H], both bf16, dominate (the tiled variant's)
+    assert rows * (768 + 2048) * 2 <= n2 < rows * (768 + 2048) * 2 + (32 << 20)
+    # the streaming variant alone keeps float rows of y for every (token, slot)
+    rc3, n3 = workspace(desc(max_tokens=8192, sched=_lib.SCHED_STREAM))
+    assert rc3 == 0 and n3 >= rows * 2048 * 4
 
 
 @pytest.mark.parametrize("kw", [
