@@ -12,6 +12,8 @@ F32, BF16 = 0, 1
 SCHED_AUTO, SCHED_STREAM, SCHED_TILED = 0, 1, 2
 FLAG_PACK_WEIGHTS = 1
 FLAG_WEIGHTS_PREPACKED = 2
+FLAG_RMSNORM = 4
+FLAG_RESIDUAL = 8
 NOALLOC_SCRATCH_BYTES = 64 << 20
 HIP_SUCCESS = 0
 HIP_ERROR_INVALID_VALUE = 1
@@ -34,6 +36,8 @@ class LayerDesc(ctypes.Structure):
         ("ffn1_weights", ctypes.c_void_p),
         ("ffn2_weights", ctypes.c_void_p),
         ("router_bias", ctypes.c_void_p),
+        ("norm_weight", ctypes.c_void_p),
+        ("norm_eps", ctypes.c_double),
     ]
 
 

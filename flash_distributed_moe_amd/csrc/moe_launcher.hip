@@ -31,6 +31,8 @@ hipError_t prepare_tiled_kernel();
 hipError_t stream_kernel_occupancy(int dtype, int* per_cu);
 hipError_t tiled_kernel_occupancy(int* per_cu);
 int tiled_max_tokens();
+hipError_t launch_rmsnorm(const void* x, const void* gamma, void* xn, int dtype, int T, int H, double eps,
+                          hipStream_t stream);
 size_t tiled_y_bytes(size_t rows, size_t hidden);
 }
 
@@ -64,7 +66,7 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct Layout {
   size_t ctl, wgflags, g1_done, tok_arrive, cand, topk_idx, topk_w, masks, word_prefix,
-      expert_count, expert_offset, perm, row_w, mtiles, h, y, pack1, pack2, total;
+      expert_count, expert_offset, perm, row_w, mtiles, h, y, xn, pack1, pack2, total;
   size_t zero_bytes;  // leading region that must be zero before a launch
   int W, max_mtiles;
 };
@@ -113,6 +115,7 @@ Layout make_layout(const FlashMoeLayerDesc& d, bool need_tiled) {
                                                      : rows;
   L.y = take(std::max(sizeof(float) * stream_rows * d.hidden,
                       need_tiled ? fmoe::tiled_y_bytes(rows, d.hidden) : 0));
+  L.xn = take((d.flags & FLASH_MOE_FLAG_RMSNORM) ? esz * static_cast<size_t>(d.max_tokens) * d.hidden : 0);
   const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
   L.pack1 = take(pack ? esz * d.experts * 2 * d.intermediate * d.hidden : 0);
   L.pack2 = take(pack ? esz * d.experts * d.hidden * d.intermediate : 0);
@@ -145,7 +148,8 @@ hipError_t validate(const FlashMoeLayerDesc* d) {
               d->max_tokens, kMaxRows / d->top_k);
   if (d->sched < FLASH_MOE_SCHED_AUTO || d->sched > FLASH_MOE_SCHED_TILED)
     FMOE_FAIL(hipErrorInvalidValue, "sched = %i", d->sched);
-  if ((d->flags & ~(FLASH_MOE_FLAG_PACK_WEIGHTS | FLASH_MOE_FLAG_WEIGHTS_PREPACKED)) != 0)
+  if ((d->flags & ~(FLASH_MOE_FLAG_PACK_WEIGHTS | FLASH_MOE_FLAG_WEIGHTS_PREPACKED |
+                    FLASH_MOE_FLAG_RMSNORM | FLASH_MOE_FLAG_RESIDUAL)) != 0)
     FMOE_FAIL(hipErrorInvalidValue, "unknown flag bits 0x%x", d->flags);
   if ((d->flags & FLASH_MOE_FLAG_PACK_WEIGHTS) && (d->flags & FLASH_MOE_FLAG_WEIGHTS_PREPACKED))
     FMOE_FAIL(hipErrorInvalidValue, "weights that are already packed need no packed copy");
@@ -249,7 +253,8 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
                 : 0;
   p.max_mtiles = L.max_mtiles;
   p.spin_limit = l->spin_limit;
-  p.tokens = tokens;
+  p.tokens = (d.flags & FLASH_MOE_FLAG_RMSNORM) ? static_cast<const void*>(l->ws + L.xn) : tokens;
+  p.residual = (d.flags & FLASH_MOE_FLAG_RESIDUAL) ? tokens : nullptr;
   p.gate = d.gate_weights;
   p.ffn1 = d.ffn1_weights;
   p.ffn2 = d.ffn2_weights;
@@ -364,6 +369,8 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
   if (desc->gate_weights == nullptr || desc->ffn1_weights == nullptr ||
       desc->ffn2_weights == nullptr)
     FMOE_FAIL(hipErrorInvalidValue, "null weight pointer");
+  if ((desc->flags & FLASH_MOE_FLAG_RMSNORM) && (desc->norm_weight == nullptr || !(desc->norm_eps >= 0.0)))
+    FMOE_FAIL(hipErrorInvalidValue, "FLASH_MOE_FLAG_RMSNORM needs norm_weight and norm_eps >= 0");
 
   FlashMoeLauncher* l = new (std::nothrow) FlashMoeLauncher();
   if (l == nullptr) FMOE_FAIL(hipErrorOutOfMemory, "host allocation failed");
@@ -446,6 +453,9 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
     FMOE_FAIL(hipErrorInvalidValue, "null tokens/output pointer");
   const fmoe::Params p = make_params(l, tokens, output, tokens_num);
   l->last_tokens = tokens_num;
+  if (l->desc.flags & FLASH_MOE_FLAG_RMSNORM)
+    FMOE_HIP_CHECK(fmoe::launch_rmsnorm(tokens, l->desc.norm_weight, l->ws + l->layout.xn, l->desc.dtype,
+                                        tokens_num, l->desc.hidden, l->desc.norm_eps, stream));
   if (flashMoeSchedFor(l, tokens_num) == FLASH_MOE_SCHED_TILED) {
     FMOE_HIP_CHECK(fmoe::launch_tiled_kernel(p, p.n_groups, stream));
   } else {
@@ -563,6 +573,12 @@ int flashMoeLaunchNoAlloc(const FlashMoeLayerDesc* desc, const void* tokens, voi
                      stream, reinterpret_cast<uint4*>(sd->ptr), n16);
   FMOE_HIP_CHECK(hipGetLastError());
   const fmoe::Params p = make_params(&l, tokens, output, tokens_num);
+  if (desc->flags & FLASH_MOE_FLAG_RMSNORM) {
+    if (desc->norm_weight == nullptr || !(desc->norm_eps >= 0.0))
+      FMOE_FAIL(hipErrorInvalidValue, "FLASH_MOE_FLAG_RMSNORM needs norm_weight and norm_eps >= 0");
+    FMOE_HIP_CHECK(fmoe::launch_rmsnorm(tokens, desc->norm_weight, l.ws + l.layout.xn, desc->dtype, tokens_num,
+                                        desc->hidden, desc->norm_eps, stream));
+  }
   if (sched == FLASH_MOE_SCHED_TILED) {
     FMOE_HIP_CHECK(fmoe::launch_tiled_kernel(p, p.n_groups, stream));
   } else {

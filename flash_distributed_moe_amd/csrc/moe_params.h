@@ -93,7 +93,8 @@ struct Params {
   int max_mtiles;
   long long spin_limit;  // bound on one dependency wait, 100 MHz ticks
 
-  const void* tokens;  // [T,H]
+  const void* tokens;  // [T,H]: what the router and the gate/up projection read (the caller's rows, or their RMSNorm)
+  const void* residual;  // [T,H] rows added to the output (the caller's rows), or null
   const void* gate;    // [E,H]
   const void* ffn1;    // [E,2I,H]  rows 0..I-1 gate proj, I..2I-1 up proj
   const void* ffn2;    // [E,H,I]

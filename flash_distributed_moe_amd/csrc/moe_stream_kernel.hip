@@ -995,6 +995,23 @@ __device__ void combine_task(ParamsRef p, int t, int chunk) {
       }
     }
     const size_t off = static_cast<size_t>(t) * p.H + c;
+    if (p.residual != nullptr) {  // output = input row + layer, the row added last
+      if constexpr (DT::EPV == 8) {
+        const unsigned long long xx = *as_global(
+            reinterpret_cast<const unsigned long long*>(reinterpret_cast<const unsigned short*>(p.residual) + off));
+        const uint2 x = make_uint2(static_cast<unsigned>(xx), static_cast<unsigned>(xx >> 32));
+        s.x += bf16_lo(x.x);
+        s.y += bf16_hi(x.x);
+        s.z += bf16_lo(x.y);
+        s.w += bf16_hi(x.y);
+      } else {
+        const uint4 x = ld16(reinterpret_cast<const float*>(p.residual) + off);
+        s.x += __uint_as_float(x.x);
+        s.y += __uint_as_float(x.y);
+        s.z += __uint_as_float(x.z);
+        s.w += __uint_as_float(x.w);
+      }
+    }
     if constexpr (DT::EPV == 8) {
       uint2 pk;
       pk.x = f2bf(s.x) | (f2bf(s.y) << 16);

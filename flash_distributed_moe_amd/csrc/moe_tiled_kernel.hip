@@ -935,6 +935,7 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
   const int H = uni(p.H), K = uni(p.K), T = uni(p.T), E = uni(p.E), W = uni(p.W);
   unsigned short* out = uni(reinterpret_cast<unsigned short*>(p.out));
   const unsigned short* y = uni(reinterpret_cast<const unsigned short*>(p.y));
+  const unsigned short* residual = uni(reinterpret_cast<const unsigned short*>(p.residual));
   const int* topk_idx = uni(p.topk_idx);
   unsigned long long* masks = uni(p.masks);
   const int tid = threadIdx.x;
@@ -983,6 +984,15 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) s[u][i] += f[i];
           }
+    }
+    if (residual != nullptr) {  // output = input row + layer, the row added last
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        float f[8];
+        unpack<BF16>(ld16(residual + static_cast<size_t>(tok[u]) * H + col[u]), f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s[u][i] += f[i];
+      }
     }
 #pragma unroll
     for (int u = 0; u < 2; ++u)

@@ -7,7 +7,7 @@
 // float32 (the reference checks for float32, pyMoeLauncherTorch.cpp:28-29);
 // `create` reads E, H, I and the dtype off the tensors and goes through
 // CreateLauncherEx, with optional top_k (default 8, the reference's compile-time
-// value), router_bias, sched and prepacked; rank / world_size other than 0 / 1
+// value), router_bias, sched, flags, norm_weight and norm_eps; rank / world_size other than 0 / 1
 // are refused. torch supplies device pointers and the current stream, nothing
 // else.
 #include <ATen/hip/HIPContext.h>
@@ -53,7 +53,8 @@ class Launcher {
 
   void create(const at::Tensor& gate, const at::Tensor& ffn1, const at::Tensor& ffn2, int max_tokens,
               const py::bytes& uid, int rank, int world_size, int top_k,
-              const c10::optional<at::Tensor>& router_bias, int sched, int flags) {
+              const c10::optional<at::Tensor>& router_bias, int sched, int flags,
+              const c10::optional<at::Tensor>& norm_weight, double norm_eps) {
     TORCH_CHECK(impl_ == nullptr, "Launcher already created");
     TORCH_CHECK(gate.defined() && ffn1.defined() && ffn2.defined(), "weight tensor is undefined");
     TORCH_CHECK(gate.dim() == 2 && ffn1.dim() == 3 && ffn2.dim() == 3,
@@ -91,6 +92,16 @@ class Launcher {
       d.router_bias = router_bias->data_ptr<float>();
       bias_ = *router_bias;
     }
+    if (flags & FLASH_MOE_FLAG_RMSNORM) {
+      TORCH_CHECK(norm_weight.has_value() && norm_weight->defined(), "FLAG_RMSNORM needs norm_weight");
+      check_tensor(*norm_weight, "norm_weight");
+      TORCH_CHECK(norm_weight->scalar_type() == gate.scalar_type() && norm_weight->dim() == 1 &&
+                      norm_weight->size(0) == hidden,
+                  "norm_weight must be [H] in the weights' dtype");
+      d.norm_weight = norm_weight->data_ptr();
+      d.norm_eps = norm_eps;
+      norm_ = *norm_weight;
+    }
     const DeviceGuard guard(gate.device());
     check_hip(CreateLauncherEx(&impl_, &d, current_stream()), "CreateLauncher");
     // the library borrows the weights: they live as long as the launcher
@@ -119,7 +130,7 @@ class Launcher {
     const DeviceGuard guard(gate_.device());
     check_hip(DestroyLauncher(impl_, current_stream()), "DestroyLauncher");
     impl_ = nullptr;
-    gate_ = ffn1_ = ffn2_ = bias_ = at::Tensor();
+    gate_ = ffn1_ = ffn2_ = bias_ = norm_ = at::Tensor();
   }
 
   bool valid() const { return impl_ != nullptr; }
@@ -134,7 +145,7 @@ class Launcher {
 
  private:
   moe::IMoeKernelLauncher* impl_ = nullptr;
-  at::Tensor gate_, ffn1_, ffn2_, bias_;
+  at::Tensor gate_, ffn1_, ffn2_, bias_, norm_;
   int64_t hidden_ = 0;
 };
 
@@ -168,6 +179,8 @@ PYBIND11_MODULE(flashMoeLauncher, m) {
   m.attr("SCHED_TILED") = static_cast<int>(FLASH_MOE_SCHED_TILED);
   m.attr("FLAG_PACK_WEIGHTS") = static_cast<int>(FLASH_MOE_FLAG_PACK_WEIGHTS);
   m.attr("FLAG_WEIGHTS_PREPACKED") = static_cast<int>(FLASH_MOE_FLAG_WEIGHTS_PREPACKED);
+  m.attr("FLAG_RMSNORM") = static_cast<int>(FLASH_MOE_FLAG_RMSNORM);
+  m.attr("FLAG_RESIDUAL") = static_cast<int>(FLASH_MOE_FLAG_RESIDUAL);
   m.def("pack_weights_in_place", &pack_weights_in_place, py::arg("ffn1_expert_weights"),
         py::arg("ffn2_expert_weights"));
   py::class_<Launcher>(m, "MoeKernelLauncher")
@@ -177,7 +190,8 @@ PYBIND11_MODULE(flashMoeLauncher, m) {
       .def("create", &Launcher::create, py::arg("gate_weights"), py::arg("ffn1_expert_weights"),
            py::arg("ffn2_expert_weights"), py::arg("max_tokens"), py::arg("uid"), py::arg("rank"),
            py::arg("world_size"), py::arg("top_k") = 8, py::arg("router_bias") = py::none(),
-           py::arg("sched") = static_cast<int>(FLASH_MOE_SCHED_AUTO), py::arg("flags") = 0)
+           py::arg("sched") = static_cast<int>(FLASH_MOE_SCHED_AUTO), py::arg("flags") = 0,
+           py::arg("norm_weight") = py::none(), py::arg("norm_eps") = 1e-6)
       .def("launch", &Launcher::launch, py::arg("tokens"), py::arg("output"))
       .def("destroy", &Launcher::destroy)
       .def_property_readonly("valid", &Launcher::valid)

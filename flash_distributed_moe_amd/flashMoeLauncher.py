@@ -61,7 +61,9 @@ class MoeKernelLauncher:
 
     def create(self, gate_weights, ffn1_expert_weights, ffn2_expert_weights, max_tokens, uid,
                rank, world_size, top_k=8, router_bias=None, sched=_lib.SCHED_AUTO,
-               pack_weights=False, prepacked=False):
+               pack_weights=False, prepacked=False, norm_weight=None, norm_eps=1e-6, residual=False):
+        """norm_weight ([H], the weights' dtype): the layer runs on rmsnorm(tokens) with this
+        weight and norm_eps; residual: the input rows are added to the output."""
         _check(self._h is None, "Launcher already created")
         for t, n in ((gate_weights, "gate_weights"), (ffn1_expert_weights, "ffn1_expert_weights"),
                      (ffn2_expert_weights, "ffn2_expert_weights")):
@@ -100,6 +102,13 @@ class MoeKernelLauncher:
         d.ffn1_weights = ffn1_expert_weights.data_ptr()
         d.ffn2_weights = ffn2_expert_weights.data_ptr()
         d.router_bias = router_bias.data_ptr() if router_bias is not None else None
+        if norm_weight is not None:
+            _check_tensor(norm_weight, "norm_weight", (gate_weights.dtype,))
+            _check(tuple(norm_weight.shape) == (hidden,), "norm_weight must be [H]")
+            d.flags |= _lib.FLAG_RMSNORM
+            d.norm_weight, d.norm_eps = norm_weight.data_ptr(), float(norm_eps)
+        if residual:
+            d.flags |= _lib.FLAG_RESIDUAL
         h = ctypes.c_void_p()
         with torch.cuda.device(gate_weights.device):
             _hip_check(self._lib.flashMoeCreate(ctypes.byref(h), ctypes.byref(d), _stream()),
@@ -108,7 +117,7 @@ class MoeKernelLauncher:
         self._dtype = gate_weights.dtype
         self._shape = (experts, hidden, inter, int(top_k))
         # weights are borrowed by the library: keep them alive with the launcher
-        self._keep = (gate_weights, ffn1_expert_weights, ffn2_expert_weights, router_bias)
+        self._keep = (gate_weights, ffn1_expert_weights, ffn2_expert_weights, router_bias, norm_weight)
         self._device = gate_weights.device
 
     @staticmethod

@@ -58,6 +58,19 @@ enum { FLASH_MOE_SCHED_AUTO = 0, FLASH_MOE_SCHED_STREAM = 1, FLASH_MOE_SCHED_TIL
  *  neither                          launches read the caller's row-major tensors. */
 enum { FLASH_MOE_FLAG_PACK_WEIGHTS = 1, FLASH_MOE_FLAG_WEIGHTS_PREPACKED = 2 };
 
+/* Optional steps at the layer's edges (neither exists in the reference, whose
+ * layer is gate + experts only, test/singleGPU/cpp/moe/reference/refFullMoe.h:9-70;
+ * with neither flag the layer computes exactly that):
+ *  FLASH_MOE_FLAG_RMSNORM   the router and the experts see rmsnorm(tokens) instead
+ *      of tokens: xn[t,k] = (x[t,k] * float(1/sqrt(mean_k x[t,k]^2 + norm_eps))) *
+ *      norm_weight[k], rounded to the layer dtype. A small kernel in front of the
+ *      layer's kernel writes xn into the workspace (+max_tokens*H elements).
+ *  FLASH_MOE_FLAG_RESIDUAL  output = tokens + layer(...): the un-normalised input
+ *      row is added to the sum over the slots (last, in float) before the one
+ *      rounding to the layer dtype. Works in place like everything else.
+ * Together: output = x + moe(rmsnorm(x)), a pre-norm transformer block's MoE half. */
+enum { FLASH_MOE_FLAG_RMSNORM = 4, FLASH_MOE_FLAG_RESIDUAL = 8 };
+
 typedef struct FlashMoeLayerDesc {
   int experts;      /* E, 1..256 */
   int hidden;       /* H, multiple of 64 */
@@ -71,6 +84,8 @@ typedef struct FlashMoeLayerDesc {
   const void* ffn1_weights;  /* device, [E,2I,H]: rows 0..I-1 gate proj, I..2I-1 up proj */
   const void* ffn2_weights;  /* device, [E,H,I] */
   const float* router_bias;  /* device, [E] float added to the logits, or NULL */
+  const void* norm_weight;   /* device, [H] in the layer dtype; read with FLASH_MOE_FLAG_RMSNORM only */
+  double norm_eps;           /* added to the mean square; read with FLASH_MOE_FLAG_RMSNORM only */
 } FlashMoeLayerDesc;
 
 /* Device bytes flashMoeCreate would allocate for this description. */

@@ -149,6 +149,42 @@ def forward(tokens, gate_w, ffn1, ffn2, k, bias=None, nthreads=None):
     return out, idx, w
 
 
+def _round_bf16(a):
+    """float32 -> nearest-even bfloat16, kept as float32."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+def rmsnorm(tokens, weight, eps, bf16=False):
+    """xn[t,k] = (x[t,k] * float32(1 / sqrt(mean_k x[t,k]^2 + eps))) * weight[k]: mean, sqrt
+    and reciprocal in float64, the two products in float32, and for bf16=True one rounding
+    to bfloat16. Not part of the reference's layer (refFullMoe.h:9-70 starts at the gate):
+    it is the definition the library's optional FLASH_MOE_FLAG_RMSNORM step is held to,
+    the usual RMSNorm (x / rms(x) * weight) with the roundings spelled out. Pinned in
+    tests/test_oracle_math.py against float64 algebra (unit-RMS rows under weight 1,
+    scale invariance, a closed-form row), not against a reference vector."""
+    x = np.ascontiguousarray(tokens, np.float32)
+    w = np.ascontiguousarray(weight, np.float32)
+    ss = np.einsum("tk,tk->t", x.astype(np.float64), x.astype(np.float64))
+    scale = (1.0 / np.sqrt(ss / np.float64(x.shape[1]) + np.float64(eps))).astype(np.float32)
+    xn = (x * scale[:, None]) * w[None, :]
+    return _round_bf16(xn) if bf16 else xn
+
+
+def layer(tokens, gate_w, ffn1, ffn2, k, bias=None, norm_weight=None, norm_eps=1e-6, residual=False,
+          bf16=False, nthreads=None):
+    """forward() with the two optional steps at its edges: the layer runs on
+    rmsnorm(tokens) when norm_weight is given, and the input rows are added to its output
+    (one float32 addition per element) when residual is set. With neither it is forward()."""
+    x = np.ascontiguousarray(tokens, np.float32)
+    xin = x if norm_weight is None else rmsnorm(x, norm_weight, norm_eps, bf16)
+    out, idx, w = forward(xin, gate_w, ffn1, ffn2, k, bias, nthreads)
+    if residual:
+        out = out + x
+    return out, idx, w
+
+
 def experts(tokens, ffn1, ffn2, topk_idx, topk_w, nthreads=None):
     tokens, tp = _f32(tokens)
     ffn1, f1p = _f32(ffn1)

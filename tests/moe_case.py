@@ -16,8 +16,9 @@ TOL = {"bf16": 1e-2, "f32": 2e-5}
 
 class GpuCase:
     def __init__(self, cfg, seed=7907, sched=_lib.SCHED_AUTO, max_tokens=None, inputs=None,
-                 pack_weights=False, prepacked=False):
+                 pack_weights=False, prepacked=False, norm_weight=None, norm_eps=1e-6, residual=False):
         self.cfg, self.seed = cfg, seed
+        self.norm_weight, self.norm_eps, self.residual = norm_weight, norm_eps, residual
         self.dev = torch.device("cuda:0")
         self.inp = inputs or synth.make_inputs_torch(cfg, seed, self.dev)
         self.launcher = MoeKernelLauncher()
@@ -25,7 +26,8 @@ class GpuCase:
         self.launcher.create(self.inp["gate"], self.inp["ffn1"], self.inp["ffn2"],
                              max_tokens or cfg.T, uid, 0, 1, top_k=cfg.k,
                              router_bias=self.inp["bias"], sched=sched,
-                             pack_weights=pack_weights, prepacked=prepacked)
+                             pack_weights=pack_weights, prepacked=prepacked,
+                             norm_weight=norm_weight, norm_eps=norm_eps, residual=residual)
 
     def run(self, tokens=None, inplace=False):
         x = self.inp["tokens"] if tokens is None else tokens
@@ -51,10 +53,17 @@ class GpuCase:
                         for k in ("gate", "ffn1", "ffn2", "bias")}
         return self._hw
 
+    def layer_input(self, x):
+        """What the router and the experts see: the rows, or their RMSNorm."""
+        if self.norm_weight is None:
+            return x
+        return oracle.rmsnorm(x, self.norm_weight.float().cpu().numpy(), self.norm_eps,
+                              bf16=self.cfg.dtype == "bf16")
+
     def check_routing(self, tokens_t, routing):
         """Bit-exact top-k indices, counts, offsets and permutation; weights to 1e-6."""
         hw = self.host_weights()
-        x = tokens_t.float().cpu().numpy()
+        x = self.layer_input(tokens_t.float().cpu().numpy())
         idx, w = oracle.gate(x, hw["gate"], self.cfg.k, bias=hw["bias"])
         assert np.array_equal(routing["topk_idx"], idx), "top-k indices differ from the oracle"
         np.testing.assert_allclose(routing["topk_w"], w, rtol=2e-6, atol=1e-7)
@@ -71,8 +80,10 @@ class GpuCase:
         got = out_t.float().cpu().numpy()
         if token_ids is not None:
             x, got = x[token_ids], got[token_ids]
-        ref, _, _ = oracle.forward(x, hw["gate"], hw["ffn1"], hw["ffn2"], self.cfg.k,
-                                   bias=hw["bias"], nthreads=nthreads)
+        gamma = None if self.norm_weight is None else self.norm_weight.float().cpu().numpy()
+        ref, _, _ = oracle.layer(x, hw["gate"], hw["ffn1"], hw["ffn2"], self.cfg.k, bias=hw["bias"],
+                                 norm_weight=gamma, norm_eps=self.norm_eps, residual=self.residual,
+                                 bf16=self.cfg.dtype == "bf16", nthreads=nthreads)
         assert np.all(np.isfinite(got)), "non-finite output"
         err = max_rel_err(got, ref)
         tol = TOL[self.cfg.dtype]

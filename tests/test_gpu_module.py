@@ -139,6 +139,21 @@ def test_python_binding_sequence_of_the_reference():
     assert launcher.valid == False  # noqa: E712
     with pytest.raises(RuntimeError, match="Launcher was destroyed"):
         launcher.launch(tokens, output)
+    # beyond the reference's surface: the pre-norm block's MoE half in one call
+    gamma = torch.linspace(0.5, 1.5, cfg.H, device=dev)
+    launcher.create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T, uniqueid, 0, 1,
+                    flags=flashMoeLauncher.FLAG_RMSNORM | flashMoeLauncher.FLAG_RESIDUAL,
+                    norm_weight=gamma, norm_eps=1e-6)
+    launcher.launch(tokens, output)
+    torch.cuda.synchronize(dev)
+    f = lambda t: t.float().cpu().numpy()
+    want = oracle.layer(f(tokens), f(inp["gate"]), f(inp["ffn1"]), f(inp["ffn2"]), cfg.k,
+                        norm_weight=f(gamma), norm_eps=1e-6, residual=True)[0]
+    assert max_rel_err(output.cpu().numpy(), want) <= 2e-5
+    with pytest.raises(RuntimeError, match="norm_weight"):
+        flashMoeLauncher.MoeKernelLauncher().create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T, uniqueid, 0, 1,
+                                                    flags=flashMoeLauncher.FLAG_RMSNORM)
+    launcher.destroy()
 
 
 def test_wrapper_packs_the_blocks_weights_in_place():

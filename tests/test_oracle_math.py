@@ -150,3 +150,64 @@ def test_synth_numpy_and_torch_agree():
     r = np.random.default_rng(0).standard_normal(10000).astype(np.float32)
     assert np.array_equal(synth.bf16_round_np(r),
                           torch.from_numpy(r).to(torch.bfloat16).float().numpy())
+
+
+def test_rmsnorm_closed_forms():
+    # a constant row a with eps = 16 - a^2: mean + eps = 16, scale = 1/4 exactly, so
+    # xn = a/4 * weight in exact arithmetic. eps added to the sum instead of the mean,
+    # or to the root instead of the mean square, gives something else.
+    H = 64
+    w = np.linspace(-2, 2, H).astype(np.float32)
+    x = np.full((1, H), 3.0, np.float32)
+    assert np.array_equal(oracle.rmsnorm(x, w, 7.0), (0.75 * w)[None, :])
+    # one-hot row of height v: mean = v^2/H, scale = sqrt(H)/|v| = 8/|v|
+    x = np.zeros((1, H), np.float32)
+    x[0, 5] = -4.0
+    want = np.zeros((1, H), np.float32)
+    want[0, 5] = -8.0 * w[5]
+    assert np.array_equal(oracle.rmsnorm(x, w, 0.0), want)
+
+
+def test_rmsnorm_against_float64_and_invariants():
+    rng = np.random.default_rng(3)
+    T, H = 9, 320
+    x = (rng.standard_normal((T, H)) * rng.uniform(0.01, 30, (T, 1))).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    eps = 1e-6
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + eps) * w
+    got = oracle.rmsnorm(x, w, eps)
+    assert got.dtype == np.float32 and np.max(np.abs(got - want) / np.abs(want)) < 3e-7
+    # weight 1, eps 0: every row comes out with unit mean square
+    unit = oracle.rmsnorm(x, np.ones(H, np.float32), 0.0).astype(np.float64)
+    assert np.allclose((unit ** 2).mean(axis=1), 1.0, atol=1e-6)
+    # a power of two on the input cancels exactly (eps = 0)
+    assert np.array_equal(oracle.rmsnorm(x * np.float32(8), w, 0.0), oracle.rmsnorm(x, w, 0.0))
+    # bf16: the nearest bfloat16 (ties to even) of the float32 result
+    import torch
+
+    rounded = oracle.rmsnorm(x, w, eps, bf16=True)
+    assert np.array_equal(rounded, torch.from_numpy(got).to(torch.bfloat16).float().numpy())
+
+
+def test_layer_edges_reduce_and_compose():
+    cfg = synth.MoeConfig("edges", 12, 64, 8, 2, 32, "f32")
+    inp = synth.make_inputs_np(cfg, 11)
+    args = (inp["gate"], inp["ffn1"], inp["ffn2"], cfg.k)
+    base, idx, wts = oracle.forward(inp["tokens"], *args)
+    plain = oracle.layer(inp["tokens"], *args)
+    assert np.array_equal(plain[0], base) and np.array_equal(plain[1], idx)
+    # zero down projection: the layer contributes nothing, the residual is the input itself
+    zero = (inp["gate"], inp["ffn1"], np.zeros_like(inp["ffn2"]), cfg.k)
+    assert np.array_equal(oracle.layer(inp["tokens"], *zero, residual=True)[0], inp["tokens"])
+    # the residual is the un-normalised row, and it is added once
+    g = np.linspace(0.5, 1.5, cfg.H).astype(np.float32)
+    both = oracle.layer(inp["tokens"], *args, norm_weight=g, norm_eps=0.0, residual=True)[0]
+    normed = oracle.layer(inp["tokens"], *args, norm_weight=g, norm_eps=0.0)[0]
+    assert np.allclose(both - normed, inp["tokens"], atol=1e-6)
+    # with the norm in front the layer no longer sees the input's scale, without it it does
+    big = inp["tokens"] * np.float32(4)
+    assert np.array_equal(oracle.layer(big, *args, norm_weight=g, norm_eps=0.0)[0], normed)
+    assert not np.array_equal(oracle.layer(big, *args)[0], base)
+    # and it sees the normalised rows: the same as handing those rows to forward()
+    assert np.array_equal(normed, oracle.forward(oracle.rmsnorm(inp["tokens"], g, 0.0), *args)[0])

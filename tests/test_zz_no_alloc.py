@@ -96,6 +96,39 @@ def test_no_alloc_equals_launcher_two_calls_in_a_row():
     assert torch.equal(g, no_alloc(big, inp_big, inp_big["tokens"], _lib.SCHED_STREAM))
 
 
+def test_no_alloc_with_norm_and_residual():
+    """The optional RMSNorm / residual steps use the static workspace too (the normalised
+    rows live there): same bits as the launcher with the same flags."""
+    dev = torch.device("cuda:0")
+    cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=40, name="decode40")
+    inp = synth.make_inputs_torch(cfg, 7907, dev)
+    gamma = synth.normal_torch(5, 9, (cfg.H,), 0.25, torch.float32, dev).add_(1.0).to(torch.bfloat16)
+    lib = _lib.load()
+    for T in (40, 7):
+        x = inp["tokens"][:T].contiguous()
+        d = layer_desc(cfg, inp, T, _lib.SCHED_AUTO)
+        d.flags = _lib.FLAG_RMSNORM | _lib.FLAG_RESIDUAL
+        d.norm_weight, d.norm_eps = gamma.data_ptr(), 1e-6
+        out = torch.full_like(x, float("nan"))
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        assert lib.flashMoeLaunchNoAlloc(ctypes.byref(d), x.data_ptr(), out.data_ptr(), T, stream) == 0
+        torch.cuda.synchronize()
+        l = MoeKernelLauncher()
+        l.create(inp["gate"], inp["ffn1"], inp["ffn2"], T, l.getDistributedUniqueId(True), 0, 1, top_k=cfg.k,
+                 router_bias=inp["bias"], norm_weight=gamma, norm_eps=1e-6, residual=True)
+        try:
+            want = torch.full_like(x, float("nan"))
+            l.launch(x, want)
+            torch.cuda.synchronize()
+        finally:
+            l.destroy()
+        assert torch.equal(out, want)
+        f = lambda t: None if t is None else t.float().cpu().numpy()
+        ref = oracle.layer(f(x), f(inp["gate"]), f(inp["ffn1"]), f(inp["ffn2"]), cfg.k, bias=f(inp["bias"]),
+                           norm_weight=f(gamma), norm_eps=1e-6, residual=True, bf16=True)[0]
+        assert max_rel_err(out.float().cpu().numpy(), ref) <= 1e-2
+
+
 def test_no_alloc_rejects_what_does_not_fit(capfd):
     dev = torch.device("cuda:0")
     cfg = synth.CONFIGS["qwen3_30b_decode"]
