@@ -184,28 +184,32 @@ __device__ __forceinline__ void load_to_lds(unsigned off, const unsigned char* b
 // --------------------------------------------------------------------- router
 // Logits as in test/singleGPU/cpp/moe/reference/refGemm.h:21-24: one chain per
 // output, k ascending, one rounding per step. The chain runs on the matrix
-// core: V_MFMA_F32_16X16X4_F32 adds its four products to the accumulator one
-// after the other in k order (checked bit for bit against a CPU fmaf chain), and
-// a product of two bf16 values is exact in float, so every step is the oracle's
-// acc = fmaf(x, w, acc). A dependent chain of these instructions runs at the
-// matrix core's full rate, so one chain per SIMD would do; a wave carries two
-// (16 tokens x experts 16w..16w+15 and 64+16w..64+16w+15 of a slab of 128), which
-// is what four waves need to cover the slab.
-// All waves load: 64 k of the 16 token rows and the 128 expert rows per stage,
+// core: V_MFMA_F32_16X16X4_F32 and V_MFMA_F32_32X32X2_F32 add their four / two
+// products to the accumulator one after the other in k order (checked bit for bit
+// against a CPU fmaf chain), and a product of two bf16 values is exact in float, so
+// every step is the oracle's acc = fmaf(x, w, acc).
+// A task is 16 or 32 tokens x a slab of 128 experts. With 16 tokens a wave carries two
+// 16x16 chains (experts 16w..16w+15 and 64+16w..64+16w+15); with 32 tokens one 32x32
+// chain (experts 32w..32w+31), which does the work of four 16x16 chains with half the
+// operand reads and permutes per multiply-add, and in less time: with every CU on the
+// float matrix core the chip holds ~56 cycles per 1024 multiply-adds in the 32x32 shape
+// against ~70 in the 16x16 shape (32 nominal for both).
+// All waves load: 64 k of the token rows and the 128 expert rows per stage,
 // four stages deep, with coalesced direct-to-LDS loads. Stage rows are 144 bytes
 // (128 of data, 16 of padding), so the 16-byte reads of 16 rows at one k fall
-// into different banks. Lane l multiplies row l % 16 of both operands at
+// into different banks. 16x16: lane l multiplies row l % 16 of both operands at
 // k = 4*s + l/16: of the eight bf16 a 16-byte read brings, elements l/16 and
-// 4 + l/16, each moved into the upper half of a zero word by one byte permute.
+// 4 + l/16. 32x32: row l % 32 at k = 2*s + l/32: elements l/32, 2 + l/32, 4 + l/32,
+// 6 + l/32. Each is moved into the upper half of a zero word by one byte permute.
 // Then selection as in refTopk.h:36-58 / refMoeGate.h:27-30.
-constexpr int RT16_TOK = 16;
+constexpr int RT16_TOK = 16;  // tokens of the small router task; the large one has twice as many
 constexpr int RT_ROW_BYTES = 144;
 constexpr int RT_STAGES = 4;
 constexpr int RT_NL = 6;                                  // loads per wave and stage
 constexpr int RT_STAGE_BYTES = WAVES * RT_NL * 1024;      // 24 KiB
-constexpr int RT_NROWS = RT16_TOK + 128;
+constexpr int RT_NROWS = 2 * RT16_TOK + 128;
 static_assert(RT_NROWS * 9 <= WAVES * RT_NL * 64, "router stage too small");
-constexpr int ROUTER_LDS_BYTES = RT_STAGES * RT_STAGE_BYTES + RT16_TOK * MAX_EXPERTS * 4 + WAVES * MAX_TOPK * 8;
+constexpr int ROUTER_LDS_BYTES = RT_STAGES * RT_STAGE_BYTES + 2 * RT16_TOK * MAX_EXPERTS * 4 + WAVES * MAX_TOPK * 8;
 
 __device__ __forceinline__ void load_to_lds_addr(const unsigned char* addr, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
@@ -214,37 +218,46 @@ __device__ __forceinline__ void load_to_lds_addr(const unsigned char* addr, unsi
                : "memory");
 }
 
+template <int NB>  // 1: 16 tokens, 16x16 chains; 2: 32 tokens, 32x32 chains
 __device__ __noinline__ void tiled_router_task(ParamsRef pv, int blk) {
+  constexpr int NTOK = NB * RT16_TOK;
+  constexpr int NROWS = NTOK + 128;
+  constexpr int NW = NB == 2 ? 1 : 2;  // expert rows a lane reads
   ParamsRef p = uniform_params(pv);
   const int T = uni(p.T), E = uni(p.E), H = uni(p.H);
   const unsigned char* tokens = uni(reinterpret_cast<const unsigned char*>(p.tokens));
   const unsigned char* gate = uni(reinterpret_cast<const unsigned char*>(p.gate));
   const float* bias = uni(p.bias);
-  unsigned* keys = reinterpret_cast<unsigned*>(lds_raw + RT_STAGES * RT_STAGE_BYTES);  // [RT16_TOK][MAX_EXPERTS]
-  double* sel = reinterpret_cast<double*>(keys + RT16_TOK * MAX_EXPERTS);              // WAVES x MAX_TOPK
+  unsigned* keys = reinterpret_cast<unsigned*>(lds_raw + RT_STAGES * RT_STAGE_BYTES);  // [NTOK][MAX_EXPERTS]
+  double* sel = reinterpret_cast<double*>(keys + NTOK * MAX_EXPERTS);              // WAVES x MAX_TOPK
   const unsigned lds_addr = uni(static_cast<unsigned>(
       reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
   const int tid = threadIdx.x;
   const int wave = uni(tid >> 6), lane = tid & 63;
-  const int t0 = uni(blk) * RT16_TOK;
+  const int t0 = uni(blk) * NTOK;
   const int nsteps = H >> 6;
   // slot g of a stage (16 bytes): position g % 9 of row g / 9 (position 8 is padding);
-  // rows 0..15 are the tokens, 16..143 the experts of the slab; slots past the last row repeat it
-  const int r16 = lane & 15, kq = lane >> 4;
-  const unsigned pick = kq == 0 ? 0x01000C0Cu : kq == 1 ? 0x03020C0Cu : kq == 2 ? 0x05040C0Cu : 0x07060C0Cu;
-  const int xoff = r16 * RT_ROW_BYTES;
-  const int woff0 = (RT16_TOK + 16 * wave + r16) * RT_ROW_BYTES;
-  const int woff1 = (RT16_TOK + 64 + 16 * wave + r16) * RT_ROW_BYTES;
+  // rows 0..NTOK-1 are the tokens, the next 128 the experts of the slab; slots past the last row repeat it
+  const int r16 = lane & 15, kq = lane >> 4;    // 16x16: row and k quarter
+  const int r32 = lane & 31, kh = lane >> 5;    // 32x32: row and k half
+  const unsigned pick = NB == 2 ? (kh == 0 ? 0x01000C0Cu : 0x03020C0Cu)
+                                : (kq == 0   ? 0x01000C0Cu
+                                   : kq == 1 ? 0x03020C0Cu
+                                   : kq == 2 ? 0x05040C0Cu
+                                             : 0x07060C0Cu);
+  const int xoff = (NB == 2 ? r32 : r16) * RT_ROW_BYTES;
+  const int woff0 = (NB == 2 ? NTOK + 32 * wave + r32 : NTOK + 16 * wave + r16) * RT_ROW_BYTES;
+  const int woff1 = (NTOK + 64 + 16 * wave + r16) * RT_ROW_BYTES;  // 16x16 only
   for (int e0 = 0; e0 < E; e0 += 128) {
     const unsigned char* src[RT_NL];
 #pragma unroll
     for (int i = 0; i < RT_NL; ++i) {
       const int g = (wave * RT_NL + i) * 64 + lane;
-      const int row = min(g / 9, RT_NROWS - 1);
+      const int row = min(g / 9, NROWS - 1);
       const int pos = min(g % 9, 7);
       const unsigned char* base =
-          row < RT16_TOK ? tokens + static_cast<size_t>(min(t0 + row, T - 1)) * H * 2
-                         : gate + static_cast<size_t>(min(e0 + row - RT16_TOK, E - 1)) * H * 2;
+          row < NTOK ? tokens + static_cast<size_t>(min(t0 + row, T - 1)) * H * 2
+                     : gate + static_cast<size_t>(min(e0 + row - NTOK, E - 1)) * H * 2;
       src[i] = base + pos * 16;
     }
     auto issue = [&](int step) {  // past the last step: the last one again, into a stage nobody reads
@@ -253,32 +266,43 @@ __device__ __noinline__ void tiled_router_task(ParamsRef pv, int blk) {
 #pragma unroll
       for (int i = 0; i < RT_NL; ++i) load_to_lds_addr(src[i] + koff, st + i * 1024);
     };
-    f32x4 acc0 = f32x4{0.f, 0.f, 0.f, 0.f}, acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};  // 16x16
+    f32x16 big;                                                               // 32x32
+#pragma unroll
+    for (int i = 0; i < 16; ++i) big[i] = 0.f;
     // Operands of half a stage (32 k): four 16-byte chunks of the token row and of the
-    // two expert rows. While the 16 matrix instructions of one half run, the next half is
-    // read, one chunk of the three rows after each four; the scheduling barriers keep the
+    // expert rows. While the 16 matrix instructions of one half run, the next half is
+    // read, one chunk of each row after every four; the scheduling barriers keep the
     // reads from being gathered in front of their first use.
     struct Half {
-      uint4 a[4], w0[4], w1[4];
+      uint4 a[4], w[NW][4];
     };
     auto read_chunk = [&](Half& h, const unsigned char* hb, int c4) {
       h.a[c4] = *reinterpret_cast<const uint4*>(hb + xoff + 16 * c4);
-      h.w0[c4] = *reinterpret_cast<const uint4*>(hb + woff0 + 16 * c4);
-      h.w1[c4] = *reinterpret_cast<const uint4*>(hb + woff1 + 16 * c4);
+      h.w[0][c4] = *reinterpret_cast<const uint4*>(hb + woff0 + 16 * c4);
+      if constexpr (NB == 1) h.w[1][c4] = *reinterpret_cast<const uint4*>(hb + woff1 + 16 * c4);
     };
+    auto sel1 = [&](unsigned v) { return __uint_as_float(__builtin_amdgcn_perm(v, v, pick)); };
     auto chain_and_read = [&](const Half& h, Half& nx, const unsigned char* nb) {
 #pragma unroll
       for (int c4 = 0; c4 < 4; ++c4) {
-        const float xl = __uint_as_float(__builtin_amdgcn_perm(h.a[c4].y, h.a[c4].x, pick));
-        const float xh = __uint_as_float(__builtin_amdgcn_perm(h.a[c4].w, h.a[c4].z, pick));
-        acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(
-            xl, __uint_as_float(__builtin_amdgcn_perm(h.w0[c4].y, h.w0[c4].x, pick)), acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(
-            xl, __uint_as_float(__builtin_amdgcn_perm(h.w1[c4].y, h.w1[c4].x, pick)), acc1, 0, 0, 0);
-        acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(
-            xh, __uint_as_float(__builtin_amdgcn_perm(h.w0[c4].w, h.w0[c4].z, pick)), acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(
-            xh, __uint_as_float(__builtin_amdgcn_perm(h.w1[c4].w, h.w1[c4].z, pick)), acc1, 0, 0, 0);
+        if constexpr (NB == 2) {
+          big = __builtin_amdgcn_mfma_f32_32x32x2f32(sel1(h.a[c4].x), sel1(h.w[0][c4].x), big, 0, 0, 0);
+          big = __builtin_amdgcn_mfma_f32_32x32x2f32(sel1(h.a[c4].y), sel1(h.w[0][c4].y), big, 0, 0, 0);
+          big = __builtin_amdgcn_mfma_f32_32x32x2f32(sel1(h.a[c4].z), sel1(h.w[0][c4].z), big, 0, 0, 0);
+          big = __builtin_amdgcn_mfma_f32_32x32x2f32(sel1(h.a[c4].w), sel1(h.w[0][c4].w), big, 0, 0, 0);
+        } else {
+          const float xl = __uint_as_float(__builtin_amdgcn_perm(h.a[c4].y, h.a[c4].x, pick));
+          const float xh = __uint_as_float(__builtin_amdgcn_perm(h.a[c4].w, h.a[c4].z, pick));
+#pragma unroll
+          for (int j = 0; j < NW; ++j)
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                xl, __uint_as_float(__builtin_amdgcn_perm(h.w[j][c4].y, h.w[j][c4].x, pick)), acc[j], 0, 0, 0);
+#pragma unroll
+          for (int j = 0; j < NW; ++j)
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                xh, __uint_as_float(__builtin_amdgcn_perm(h.w[j][c4].w, h.w[j][c4].z, pick)), acc[j], 0, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
         read_chunk(nx, nb, c4);
         __builtin_amdgcn_sched_barrier(0);
@@ -305,26 +329,38 @@ __device__ __noinline__ void tiled_router_task(ParamsRef pv, int blk) {
     wait_vm<0>();                  // nothing may land in a stage after this slab
     __builtin_amdgcn_s_barrier();  // the stages may be refilled for the next slab
     asm volatile("" ::: "memory");
-    // acc[v] of lane l: token 4*(l/16) + v, expert e0 + (0 | 64) + 16*wave + l%16
-    const int ea = e0 + 16 * wave + r16, eb = ea + 64;
-    const float bva = (bias != nullptr && ea < E) ? as_global(bias)[ea] : 0.0f;
-    const float bvb = (bias != nullptr && eb < E) ? as_global(bias)[eb] : 0.0f;
+    if constexpr (NB == 2) {
+      // big[i] of lane l: token 8*(i/4) + 4*(l/32) + i%4, expert e0 + 32*wave + l%32
+      const int e = e0 + 32 * wave + r32;
+      const float bv = (bias != nullptr && e < E) ? as_global(bias)[e] : 0.0f;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      float xa = acc0[v], xb = acc1[v];
-      if (bias != nullptr) {
-        xa = __fadd_rn(xa, bva);
-        xb = __fadd_rn(xb, bvb);
+      for (int i = 0; i < 16; ++i) {
+        const float x = bias != nullptr ? __fadd_rn(big[i], bv) : big[i];
+        const int tl = 8 * (i >> 2) + 4 * kh + (i & 3);
+        if (e < MAX_EXPERTS) keys[tl * MAX_EXPERTS + e] = ordered_bits(x, e < E);
       }
-      if (ea < MAX_EXPERTS) keys[(4 * kq + v) * MAX_EXPERTS + ea] = ordered_bits(xa, ea < E);
-      if (eb < MAX_EXPERTS) keys[(4 * kq + v) * MAX_EXPERTS + eb] = ordered_bits(xb, eb < E);
+    } else {
+      // acc[j][v] of lane l: token 4*(l/16) + v, expert e0 + 64*j + 16*wave + l%16
+      const int ea = e0 + 16 * wave + r16, eb = ea + 64;
+      const float bva = (bias != nullptr && ea < E) ? as_global(bias)[ea] : 0.0f;
+      const float bvb = (bias != nullptr && eb < E) ? as_global(bias)[eb] : 0.0f;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        float xa = acc[0][v], xb = acc[1][v];
+        if (bias != nullptr) {
+          xa = __fadd_rn(xa, bva);
+          xb = __fadd_rn(xb, bvb);
+        }
+        if (ea < MAX_EXPERTS) keys[(4 * kq + v) * MAX_EXPERTS + ea] = ordered_bits(xa, ea < E);
+        if (eb < MAX_EXPERTS) keys[(4 * kq + v) * MAX_EXPERTS + eb] = ordered_bits(xb, eb < E);
+      }
     }
   }
   __syncthreads();
-  // selection: four tokens per wave
+  // selection: every wave takes its share of the tokens
   double* lex = sel + wave * MAX_TOPK;
-  for (int i = 0; i < RT16_TOK / WAVES; ++i) {
-    const int tl = wave * (RT16_TOK / WAVES) + i;
+  for (int i = 0; i < NTOK / WAVES; ++i) {
+    const int tl = wave * (NTOK / WAVES) + i;
     const int t = t0 + tl;
     if (t < T) {
       unsigned val[MAX_EXPERTS / 64];
@@ -930,6 +966,10 @@ constexpr int TILED_LDS_BYTES =
 
 // combine: out[t] = sum over slots, in slot order, of y[t*K+slot]
 // (refFullMoe.h:35,62-65).
+#ifndef FMOE_CMB_U
+#define FMOE_CMB_U 4
+#endif
+constexpr int CMB_U = FMOE_CMB_U;  // items a thread of the combine task has in flight
 __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
   ParamsRef p = uniform_params(pv);
   const int H = uni(p.H), K = uni(p.K), T = uni(p.T), E = uni(p.E), W = uni(p.W);
@@ -945,18 +985,18 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
   unsigned char* flag = lds_raw;  // [CMB_TOK * MAX_TOPK]
   if (tid < ntok * K) flag[tid] = ldc(&topk_idx[static_cast<size_t>(t0) * K + tid]) >= 0 ? 1 : 0;
   __syncthreads();
-  // one item = 8 columns of one token; a thread works on two items at a time, so that 2*K
-  // row loads are in flight per lane (one CU alone needs about 64 KiB in flight for its share
-  // of the memory bandwidth)
+  // one item = 8 columns of one token; a thread works on CMB_U items at a time, so that
+  // CMB_U*K row loads are in flight per lane (one CU alone needs about 64 KiB in flight for
+  // its share of the memory bandwidth)
   const int cpr = H >> 3;  // items per token
   const int nitems = ntok * cpr;
-  for (int it0 = tid; it0 < nitems; it0 += 2 * T_THREADS) {
-    float s[2][8];
-    unsigned valid[2];
-    const unsigned short* yrow[2];
-    int tok[2], col[2];
+  for (int it0 = tid; it0 < nitems; it0 += CMB_U * T_THREADS) {
+    float s[CMB_U][8];
+    unsigned valid[CMB_U];
+    const unsigned short* yrow[CMB_U];
+    int tok[CMB_U], col[CMB_U];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < CMB_U; ++u) {
       const int it = min(it0 + u * T_THREADS, nitems - 1);
       const int tl = it / cpr;
       col[u] = (it - tl * cpr) << 3;
@@ -968,14 +1008,14 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
       for (int i = 0; i < 8; ++i) s[u][i] = 0.0f;
     }
     for (int k0 = 0; k0 < K; k0 += 8) {
-      uint4 v[2][8];
+      uint4 v[CMB_U][8];
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < CMB_U; ++u)
 #pragma unroll
         for (int k = 0; k < 8; ++k)
           if (k0 + k < K) v[u][k] = ld16_once(yrow[u] + static_cast<size_t>(k0 + k) * H);
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < CMB_U; ++u)
 #pragma unroll
         for (int k = 0; k < 8; ++k)
           if (k0 + k < K && ((valid[u] >> (k0 + k)) & 1u)) {
@@ -987,7 +1027,7 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
     }
     if (residual != nullptr) {  // output = input row + layer, the row added last
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < CMB_U; ++u) {
         float f[8];
         unpack<BF16>(ld16(residual + static_cast<size_t>(tok[u]) * H + col[u]), f);
 #pragma unroll
@@ -995,7 +1035,7 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
       }
     }
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int u = 0; u < CMB_U; ++u)
       if (it0 + u * T_THREADS < nitems)
         st16(out + static_cast<size_t>(tok[u]) * H + col[u],
              u32x4{pack_bf16(s[u][0], s[u][1]), pack_bf16(s[u][2], s[u][3]), pack_bf16(s[u][4], s[u][5]),
@@ -1040,7 +1080,11 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
   Control* ctl = p.ctl;
   const unsigned T = static_cast<unsigned>(p.T);
   const unsigned n_sc = (T + RT_TOK - 1u) / RT_TOK;  // scatter tasks
-  const unsigned n_rt = (T + RT16_TOK - 1u) / RT16_TOK;  // router tasks
+  // router tasks: 16 tokens each while one round of them covers the batch, 32 beyond that
+  // (a task of 32 takes longer than one of 16, but less than two of them)
+  const bool rt2 = (T + RT16_TOK - 1u) / RT16_TOK > gridDim.x;
+  const unsigned rt_tok = rt2 ? 2u * RT16_TOK : 1u * RT16_TOK;
+  const unsigned n_rt = (T + rt_tok - 1u) / rt_tok;
   const unsigned n_es = (static_cast<unsigned>(p.E) + SCAN_EXPERTS - 1u) / SCAN_EXPERTS;
   const unsigned t_escan0 = n_rt;
   const unsigned t_scan = n_rt + n_es;
@@ -1083,7 +1127,11 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
     long long t_ready = 0;
     if (tk < n_rt) {
       if (p.trace) t_ready = wall_clock64();
-      tiled_router_task(p, static_cast<int>(tk));
+      if (rt2) {
+        tiled_router_task<2>(p, static_cast<int>(tk));
+      } else {
+        tiled_router_task<1>(p, static_cast<int>(tk));
+      }
       wg_arrive<false>(&ctl->router_done.v, &sh);
       trace(tk, 0, tk, t_fetch, t_ready);
     } else if (tk < t_scan) {
@@ -1152,15 +1200,8 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
         const unsigned m = lo + j / nt1;
         if (p.trace) t_ready = wall_clock64();
         const TileDesc tile = ld_tile(&p.mtiles[m]);
-#ifdef FMOE_X_SYNC
-        fence_release();
-        __syncthreads();
-#endif
         tiled_gemm_task(p, tile, static_cast<int>(j % nt1), 0, pend, &ctl->xq[q].v);
         pend = &p.g1_done[m].v;
-#ifdef FMOE_X_FLUSH
-        flush();
-#endif
         trace(t_dyn0 + lo * nt1 + j, 3, m, t_fetch, t_ready);
         j = task_notes()[0];
       } else {
@@ -1177,15 +1218,8 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
         ok = wg_wait_ge(p, &p.g1_done[m].v, nt1, &sh);
         if (ok) {
           if (p.trace) t_ready = wall_clock64();
-#ifdef FMOE_X_SYNC
-          fence_release();
-          __syncthreads();
-#endif
           tiled_gemm_task(p, tile, static_cast<int>(jj % nt2), 1, pend, &ctl->xq[q].v);
           pend = &ctl->g2_done.v;
-#ifdef FMOE_X_FLUSH
-          flush();
-#endif
           trace(t_dyn0 + nm * nt1 + lo * nt2 + jj, 4, m, t_fetch, t_ready);
           j = task_notes()[0];
         }
