@@ -746,10 +746,12 @@ __device__ __forceinline__ unsigned packed_run_offset(int q) {
 // matching up rows, so SiLU(gate)*up happens in registers; the tile's 128 columns leave
 // through LDS as 256-byte row segments.
 //
-// down: y[t*K+slot, n0 .. n0+256) = w * (h[row] . W2[e]^T) (refFullMoe.h:58-65,
+// down: y[t*K+slot, n0 .. n0+256) = h[row] . W2[e]^T (refFullMoe.h:58-65,
 // src/hip/kernel/tasks/ffn2Task.h:37-40), bf16, through LDS as 512-byte row segments, 128
-// rows at a time. The rows' destinations and gate weights are fetched when the task starts
-// and parked in LDS behind the stages, so the epilogue waits for no memory.
+// rows at a time. The rows' destinations are fetched when the task starts and parked in LDS
+// behind the stages, so the epilogue waits for no memory. The slot's gate weight is applied
+// by the combine task, which has instruction slots to spare; here every instruction of the
+// epilogue is one the matrix cores wait for.
 template <int JT, bool down>
 __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int rows, int nblk, unsigned* pend,
                                           unsigned* queue) {
@@ -763,7 +765,6 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
   const int n0 = uni(nblk) * (down ? TN : G1_COLS);
   TileOperands op;
   int side_dst[2];
-  float side_w[2];
   int nstages;
   if (down) {
     nstages = I / KS;
@@ -779,12 +780,10 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
       op.wstride = static_cast<unsigned>(ROWB);
     }
     op.tbase = uni(reinterpret_cast<const unsigned char*>(p.h)) + static_cast<size_t>(row0) * I * 2;
-    const float* row_w = uni(p.row_w) + row0;
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const int r = static_cast<int>(threadIdx.x) + k * T_THREADS;
       side_dst[k] = r < rows ? ldc(&perm[r]) : -1;
-      side_w[k] = r < rows ? ldc(&row_w[r]) : 0.0f;
     }
 #pragma unroll
     for (int q = 0; q < NLD; ++q) {
@@ -882,14 +881,10 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
     __syncthreads();  // the slab is stage memory again
   } else {
     int* sdst = reinterpret_cast<int*>(lds_raw + SIDE_OFF);
-    float* sw = reinterpret_cast<float*>(lds_raw + SIDE_OFF + TM_MAX * 4);
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const int r = static_cast<int>(threadIdx.x) + k * T_THREADS;
-      if (r < TM_MAX) {
-        sdst[r] = side_dst[k];
-        sw[r] = side_w[k];
-      }
+      if (r < TM_MAX) sdst[r] = side_dst[k];
     }
     __syncthreads();
     unsigned char* y = uni(reinterpret_cast<unsigned char*>(p.y)) + n0 * 2;
@@ -899,14 +894,13 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
       for (int jj = 0; jj < 4; ++jj) {
         const int j = part * 4 + jj;
         if (j < JT) {
-          const float w = sw[j * 32 + r32];
 #pragma unroll
           for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
               uint2 pk;
-              pk.x = pack_bf16(acc[i][j][g4 * 4 + 0] * w, acc[i][j][g4 * 4 + 1] * w);
-              pk.y = pack_bf16(acc[i][j][g4 * 4 + 2] * w, acc[i][j][g4 * 4 + 3] * w);
+              pk.x = pack_bf16(acc[i][j][g4 * 4 + 0], acc[i][j][g4 * 4 + 1]);
+              pk.y = pack_bf16(acc[i][j][g4 * 4 + 2], acc[i][j][g4 * 4 + 3]);
               *reinterpret_cast<uint2*>(slab + (jj * 32 + r32) * EPI_LD +
                                         (wave * 64 + i * 32 + g4 * 8 + kq * 4) * 2) = pk;
             }
@@ -964,8 +958,9 @@ __device__ __noinline__ void tiled_gemm_task(ParamsRef pv, const TileDesc& tile_
 constexpr int TILED_LDS_BYTES =
     NOTE_OFF + NOTE_BYTES > ROUTER_LDS_BYTES ? NOTE_OFF + NOTE_BYTES : ROUTER_LDS_BYTES;
 
-// combine: out[t] = sum over slots, in slot order, of y[t*K+slot]
-// (refFullMoe.h:35,62-65).
+// combine: out[t] = sum over slots, in slot order, of w[t,slot] * y[t*K+slot]
+// (refFullMoe.h:35,62-65): y holds each slot's down-projection row rounded to bf16; weight
+// and sum are float, one fused multiply-add per slot, then one rounding to bf16.
 #ifndef FMOE_CMB_U
 #define FMOE_CMB_U 4
 #endif
@@ -977,13 +972,18 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
   const unsigned short* y = uni(reinterpret_cast<const unsigned short*>(p.y));
   const unsigned short* residual = uni(reinterpret_cast<const unsigned short*>(p.residual));
   const int* topk_idx = uni(p.topk_idx);
+  const float* topk_w = uni(p.topk_w);
   unsigned long long* masks = uni(p.masks);
   const int tid = threadIdx.x;
   const int t0 = uni(blk) * CMB_TOK;
   const int ntok = min(CMB_TOK, T - t0);
-  // which (token, slot) pairs of this task hold an expert: one load each
-  unsigned char* flag = lds_raw;  // [CMB_TOK * MAX_TOPK]
-  if (tid < ntok * K) flag[tid] = ldc(&topk_idx[static_cast<size_t>(t0) * K + tid]) >= 0 ? 1 : 0;
+  // which (token, slot) pairs of this task hold an expert, and their gate weights: one load each
+  float* wts = reinterpret_cast<float*>(lds_raw);                      // [CMB_TOK * MAX_TOPK]
+  unsigned char* flag = lds_raw + CMB_TOK * MAX_TOPK * sizeof(float);  // [CMB_TOK * MAX_TOPK]
+  if (tid < ntok * K) {
+    flag[tid] = ldc(&topk_idx[static_cast<size_t>(t0) * K + tid]) >= 0 ? 1 : 0;
+    wts[tid] = ldc(&topk_w[static_cast<size_t>(t0) * K + tid]);
+  }
   __syncthreads();
   // one item = 8 columns of one token; a thread works on CMB_U items at a time, so that
   // CMB_U*K row loads are in flight per lane (one CU alone needs about 64 KiB in flight for
@@ -994,11 +994,13 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
     float s[CMB_U][8];
     unsigned valid[CMB_U];
     const unsigned short* yrow[CMB_U];
+    const float* wrow[CMB_U];
     int tok[CMB_U], col[CMB_U];
 #pragma unroll
     for (int u = 0; u < CMB_U; ++u) {
       const int it = min(it0 + u * T_THREADS, nitems - 1);
       const int tl = it / cpr;
+      wrow[u] = wts + tl * K;
       col[u] = (it - tl * cpr) << 3;
       tok[u] = t0 + tl;
       valid[u] = 0u;
@@ -1021,8 +1023,9 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
           if (k0 + k < K && ((valid[u] >> (k0 + k)) & 1u)) {
             float f[8];
             unpack<BF16>(v[u][k], f);
+            const float w = wrow[u][k0 + k];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) s[u][i] += f[i];
+            for (int i = 0; i < 8; ++i) s[u][i] = __fmaf_rn(f[i], w, s[u][i]);
           }
     }
     if (residual != nullptr) {  // output = input row + layer, the row added last
@@ -1047,7 +1050,7 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
       for (int e = tid; e < E; e += T_THREADS) stc(&masks[static_cast<size_t>(e) * W + (t >> 6)], 0ull);
     }
   }
-  __syncthreads();  // flag[] is reused by the next task
+  __syncthreads();  // flag[] and wts[] are reused by the next task
 }
 // ---------------------------------------------------------------- worker loop
 // Ticket layout. The prologue (router, scan, scatter) uses one global counter.
