@@ -238,6 +238,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy 1 GiB device to device five times: the known traffic the "
                          "rocprofv3 byte counters are scaled by")
+    ap.add_argument("--gemm-calibration", action="store_true",
+                    help="time torch.matmul (the vendor GEMM) in bf16 on this box: the matrix-core "
+                         "rate reachable in practice, next to the published peak")
     ap.add_argument("--record-traffic", nargs=2, type=float, metavar=("FETCH_KIB", "WRITE_KIB"),
                     help="no GPU work: write the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings "
                          "(KiB per dispatch) of --config into profiles/traffic.json")
@@ -266,6 +269,33 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"copies": 5, "kib_read_each": 1 << 20,
                                                "kib_written_each": 1 << 20}}))
+        return
+
+    if args.gemm_calibration:
+        # What the vendor's GEMM (torch.matmul -> hipBLASLt) reaches on this box, on operands of
+        # the same kind (bf16, normal random values): the matrix-core ceiling a kernel meets in
+        # practice here, to set beside the published peak the roofline is quoted against.
+        out = {}
+        for name, (m, n, k) in {"square_8192": (8192, 8192, 8192),
+                                "layer_gate_up_as_one_gemm": (65536, 1536, 2048),
+                                "layer_down_as_one_gemm": (65536, 2048, 768)}.items():
+            a = torch.randn(m, k, device="cuda:0", dtype=torch.bfloat16)
+            b = torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02
+            for _ in range(5):
+                torch.matmul(a, b.t())
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = 30
+            e0.record()
+            for _ in range(reps):
+                torch.matmul(a, b.t())
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            out[name] = {"m": m, "n": n, "k": k, "us": us, "tflops": 2.0 * m * n * k / us / 1e6,
+                         "frac_of_2500": 2.0 * m * n * k / us / 1e6 / 2500.0}
+            del a, b
+        print(json.dumps({"gemm_calibration": out}))
         return
 
     cfg, inp, ms_per_step, roofline, config = measure(args.config, args.seed, args.steps,
