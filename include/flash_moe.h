@@ -132,14 +132,16 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
  * kernels and results as flashMoeCreate + flashMoeLaunch on the same inputs, but
  * the workspace is a static device array of FLASH_MOE_NOALLOC_SCRATCH_BYTES that
  * every device the library runs on holds until the process ends. `desc` is read
- * as in flashMoeCreate (weights borrowed for the duration of the launch; flags
- * must be 0: there is no packed weight copy); the workspace is laid out for
- * tokens_num alone, and with FLASH_MOE_SCHED_AUTO the variant is the one
- * flashMoeLaunch would take if its workspace fits, else the streaming one.
+ * as in flashMoeCreate (weights borrowed for the duration of the launch; every
+ * flag but FLASH_MOE_FLAG_PACK_WEIGHTS is honoured: the array has no room for a
+ * packed weight copy, weights the caller has packed in place are fine); the
+ * workspace is laid out for tokens_num alone, and with FLASH_MOE_SCHED_AUTO the
+ * variant is the one flashMoeLaunch would take if its workspace fits, else the
+ * streaming one.
  * hipErrorUnknown when tokens_num > desc->max_tokens or when that batch needs
- * more workspace than the array holds (it holds about 700 tokens of the
- * E128/H2048/I768/top-8 bf16 shape and 300 of E128/H4096/I1536/top-8 with the
- * streaming variant); nothing is enqueued then.
+ * more workspace than the array holds (bf16, top-8, 128 experts: 847 tokens of
+ * the H2048/I768 shape with the streaming variant and 1447 with the tiled one,
+ * 426 and 733 of H4096/I1536); nothing is enqueued then.
  * Enqueues a small clearing kernel and the layer's kernel on `stream`, waits
  * for nothing, calls no hipMalloc/hipFree. The first call on a device looks up
  * the array's address and the device's properties (make it outside a graph

@@ -182,7 +182,16 @@ def test_tiled_variant_forced(shape):
             r1, r2 = case.launcher.routing(T), other.launcher.routing(T)
             assert np.array_equal(r1["topk_idx"], r2["topk_idx"])
             assert np.array_equal(r1["perm"], r2["perm"])
-            assert torch.allclose(out.float(), out2.float(), rtol=2e-2, atol=1e-3)
+            # Outputs: the streaming variant sums float rows and rounds once; the tiled one
+            # rounds each slot's down-projection row to bf16 first (relative 2^-9 each, the
+            # weights sum to 1), then both round the sum to bf16. Per token the two may
+            # therefore differ by a few bf16 ulps (2^-7 relative) of the row's largest
+            # element, and by no more.
+            a, b = out.float(), out2.float()
+            ulp = a.abs().max(dim=1, keepdim=True).values * 2.0 ** -7
+            worst = float(((a - b).abs() / ulp).max())
+            print("  tiled vs streaming: %.2f bf16 ulps of the row maximum" % worst, flush=True)
+            assert worst <= 3.0
         finally:
             other.close()
         # the tiled variant reading the packed weight copy computes the same bits
