@@ -185,13 +185,13 @@ def test_tiled_variant_forced(shape):
             # Outputs: the streaming variant sums float rows and rounds once; the tiled one
             # rounds each slot's down-projection row to bf16 first (relative 2^-9 each, the
             # weights sum to 1), then both round the sum to bf16. Per token the two may
-            # therefore differ by a few bf16 ulps (2^-7 relative) of the row's largest
+            # therefore differ by a bf16 ulp or two (2^-7 relative) of the row's largest
             # element, and by no more.
             a, b = out.float(), out2.float()
             ulp = a.abs().max(dim=1, keepdim=True).values * 2.0 ** -7
             worst = float(((a - b).abs() / ulp).max())
             print("  tiled vs streaming: %.2f bf16 ulps of the row maximum" % worst, flush=True)
-            assert worst <= 3.0
+            assert worst <= 2.0          # measured: at most 1.00
         finally:
             other.close()
         # the tiled variant reading the packed weight copy computes the same bits
