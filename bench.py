@@ -98,8 +98,12 @@ def algorithmic_flops(cfg):
 
 
 def cpu_baseline(cfg, inp, seconds_budget=25.0):
-    """The CPU oracle (restatement of the reference's CPU MoE, one thread, as the
-    reference ships it) on a bounded sample of the same workload."""
+    """The reference's CPU MoE on a bounded sample of the same workload, one thread, as the
+    reference ships it: the reference's own headers compiled behind C entry points
+    (oracle/_ref, kind "reference") where that library has been built and the workload is one
+    it covers (no router bias), else the restatement of it (kind "port"; the two return the
+    same bits, tests/test_oracle_vs_ref.py). The restatement with the tokens dealt out over
+    all host cores is reported beside it."""
     from oracle import oracle
 
     gate = inp["gate"].float().cpu().numpy()
@@ -107,18 +111,25 @@ def cpu_baseline(cfg, inp, seconds_budget=25.0):
     ffn2 = inp["ffn2"].float().cpu().numpy()
     bias = None if inp["bias"] is None else inp["bias"].float().cpu().numpy()
     x = inp["tokens"].float().cpu().numpy()
+    use_ref = bias is None and oracle.have_ref()
+
+    def one_thread(rows):
+        if use_ref:
+            return oracle.ref_full_moe(rows, gate, ffn1, ffn2, cfg.k)
+        return oracle.forward(rows, gate, ffn1, ffn2, cfg.k, bias=bias, nthreads=1)[0]
+
     # cost is linear in tokens: time 2 tokens, then size the sample to the budget
     t0 = time.perf_counter()
-    oracle.forward(x[:2], gate, ffn1, ffn2, cfg.k, bias=bias, nthreads=1)
+    one_thread(x[:2])
     per_tok = (time.perf_counter() - t0) / 2
     n = int(max(2, min(cfg.T, seconds_budget / max(per_tok, 1e-9))))
     # repeat the sample until about 10 s of CPU work have been timed
     reps = int(max(1, min(50, 10.0 / max(per_tok * n, 1e-9))))
     t0 = time.perf_counter()
     for _ in range(reps):
-        oracle.forward(x[:n], gate, ffn1, ffn2, cfg.k, bias=bias, nthreads=1)
+        one_thread(x[:n])
     dt = (time.perf_counter() - t0) / reps
-    # the same oracle with the tokens dealt out over all host cores (tokens are independent)
+    # the restatement with the tokens dealt out over all host cores (tokens are independent)
     cores = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or 64))
     m = int(min(cfg.T, max(n, 4 * cores)))
     t0 = time.perf_counter()
@@ -128,11 +139,11 @@ def cpu_baseline(cfg, inp, seconds_budget=25.0):
         "value": n / dt,
         "unit": "tokens/s",
         "cores": 1,
-        "kind": "port",
+        "kind": "reference" if use_ref else "port",
         "sample": "first %d of %d tokens of the workload, %d passes of %.2f s, one thread"
                   % (n, cfg.T, reps, dt),
         "us_per_layer_extrapolated": dt / n * cfg.T * 1e6,
-        "all_cores": {"value": m / dt_all, "unit": "tokens/s", "cores": cores,
+        "all_cores": {"value": m / dt_all, "unit": "tokens/s", "cores": cores, "kind": "port",
                       "sample": "first %d tokens, one pass of %.2f s, tokens sharded over %d threads"
                                 % (m, dt_all, cores)},
     }
