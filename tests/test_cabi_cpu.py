@@ -62,6 +62,23 @@ def test_workspace_size_grows_with_tokens():
     assert rc3 == 0 and n3 >= rows * 2048 * 4
 
 
+def test_workspace_of_the_optional_steps_and_weight_modes():
+    base = workspace(desc(max_tokens=4096))[1]
+    # the normalised rows live in the workspace: max_tokens x H elements, no more
+    with_norm = workspace(desc(max_tokens=4096, flags=_lib.FLAG_RMSNORM))[1]
+    assert 4096 * 2048 * 2 <= with_norm - base < 4096 * 2048 * 2 + 4096
+    # the residual needs nothing; weights the caller packed in place need nothing either
+    assert workspace(desc(max_tokens=4096, flags=_lib.FLAG_RESIDUAL))[1] == base
+    assert workspace(desc(max_tokens=64, flags=_lib.FLAG_WEIGHTS_PREPACKED))[1] == workspace(desc())[1]
+    # the launcher's own packed copy is the size of the expert weights
+    copy = workspace(desc(flags=_lib.FLAG_PACK_WEIGHTS))[1] - workspace(desc())[1]
+    assert 3 * 128 * 2048 * 768 * 2 <= copy < 3 * 128 * 2048 * 768 * 2 + 4096
+    # unknown flag bits, and the two weight modes together, are refused
+    assert workspace(desc(flags=16))[0] == _lib.HIP_ERROR_INVALID_VALUE
+    assert workspace(desc(flags=_lib.FLAG_PACK_WEIGHTS | _lib.FLAG_WEIGHTS_PREPACKED))[0] == \
+        _lib.HIP_ERROR_INVALID_VALUE
+
+
 @pytest.mark.parametrize("kw", [
     dict(experts=0), dict(experts=257), dict(top_k=0), dict(top_k=129), dict(top_k=33),
     dict(hidden=2000), dict(hidden=0), dict(intermediate=100), dict(dtype=7),
