@@ -527,6 +527,8 @@ int flashMoeLaunchNoAlloc(const FlashMoeLayerDesc* desc, const void* tokens, voi
   if (desc->gate_weights == nullptr || desc->ffn1_weights == nullptr ||
       desc->ffn2_weights == nullptr)
     FMOE_FAIL(hipErrorInvalidValue, "null weight pointer");
+  if ((desc->flags & FLASH_MOE_FLAG_RMSNORM) && (desc->norm_weight == nullptr || !(desc->norm_eps >= 0.0)))
+    FMOE_FAIL(hipErrorInvalidValue, "FLASH_MOE_FLAG_RMSNORM needs norm_weight and norm_eps >= 0");
   if (tokens_num < 0) FMOE_FAIL(hipErrorInvalidValue, "tokens_num = %i", tokens_num);
   if (tokens_num > desc->max_tokens)
     FMOE_FAIL(hipErrorUnknown, "tokens_num = %i exceeds max_tokens = %i", tokens_num,
@@ -573,12 +575,9 @@ int flashMoeLaunchNoAlloc(const FlashMoeLayerDesc* desc, const void* tokens, voi
                      stream, reinterpret_cast<uint4*>(sd->ptr), n16);
   FMOE_HIP_CHECK(hipGetLastError());
   const fmoe::Params p = make_params(&l, tokens, output, tokens_num);
-  if (desc->flags & FLASH_MOE_FLAG_RMSNORM) {
-    if (desc->norm_weight == nullptr || !(desc->norm_eps >= 0.0))
-      FMOE_FAIL(hipErrorInvalidValue, "FLASH_MOE_FLAG_RMSNORM needs norm_weight and norm_eps >= 0");
+  if (desc->flags & FLASH_MOE_FLAG_RMSNORM)
     FMOE_HIP_CHECK(fmoe::launch_rmsnorm(tokens, desc->norm_weight, l.ws + l.layout.xn, desc->dtype, tokens_num,
                                         desc->hidden, desc->norm_eps, stream));
-  }
   if (sched == FLASH_MOE_SCHED_TILED) {
     FMOE_HIP_CHECK(fmoe::launch_tiled_kernel(p, p.n_groups, stream));
   } else {
