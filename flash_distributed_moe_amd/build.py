@@ -20,11 +20,6 @@ HIPCC_FLAGS = [
 ]
 
 
-def extra_flags():
-    """Extra hipcc flags from the environment (timing experiments: -DFMOE_DBG_...)."""
-    return os.environ.get("FLASH_MOE_HIPCC_FLAGS", "").split()
-
-
 def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
@@ -37,7 +32,7 @@ def build(verbose=True):
     for src in sources():
         obj = os.path.join(LIB_DIR, os.path.basename(src) + ".o")
         objs.append(obj)
-        cmd = [hipcc] + HIPCC_FLAGS + extra_flags() + ["-c", src, "-o", obj]
+        cmd = [hipcc] + HIPCC_FLAGS + ["-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((cmd, subprocess.Popen(cmd, stderr=subprocess.PIPE, text=True)))

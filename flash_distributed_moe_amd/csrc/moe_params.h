@@ -18,14 +18,8 @@ enum : unsigned {
 constexpr int SKINNY_MT = 64;
 // Widths of one wave task: gate/up task = 32 gate + 32 up weight rows,
 // down task = 64 weight rows.
-#ifndef FMOE_G1_NB
-#define FMOE_G1_NB 2
-#endif
-#ifndef FMOE_G2_NB
-#define FMOE_G2_NB 4
-#endif
-constexpr int G1_NB = FMOE_G1_NB;  // 16-wide column blocks per gate/up wave task
-constexpr int G2_NB = FMOE_G2_NB;  // 16-wide column blocks per down wave task
+constexpr int G1_NB = 2;  // 16-wide column blocks per gate/up wave task
+constexpr int G2_NB = 4;  // 16-wide column blocks per down wave task
 // Output columns summed by one combine task.
 constexpr int COMBINE_COLS = 256;
 constexpr int ROUTER_TOK = 8;    // streaming variant: tokens per router dot task

@@ -513,7 +513,7 @@ constexpr int TILE_LDS_BYTES = 2 * stage_bytes_of(JT_MAX);          // 147456
 constexpr int SIDE_OFF = TILE_LDS_BYTES;
 constexpr int SIDE_BYTES = TM_MAX * 8;
 // and behind those one 16-byte line of words a GEMM task leaves for the worker loop: the ticket it
-// drew for the workgroup's next task, and (timing experiments) its phase times. They live in
+// drew for the workgroup's next task. They live in
 // the dynamic block because a file-scope LDS variable written from a function that is not
 // inlined landed on top of the dynamic block's first bytes.
 constexpr int NOTE_OFF = SIDE_OFF + SIDE_BYTES;
@@ -725,6 +725,267 @@ __device__ __forceinline__ void tile_gemm(const TileOperands& op, int nstages, f
   __syncthreads();  // the stages are free for the epilogue
 }
 
+// The same product when the weights come from the packed layout, on a deeper pipeline that
+// keeps its depth in registers instead of LDS.
+//
+// A wave's 64 weight rows are its own: no other wave reads them. So they do not go through
+// LDS at all: every fragment (32 rows x 16 k, 16 bytes per lane) is one global load straight
+// into the registers the matrix instruction reads, four 256-byte segments of the packed runs
+// per instruction. Two register sets: the fragments of stage s+2 are requested into the
+// registers of stage s as soon as its sub-step is through, two stages (about 2 us) before
+// they are needed. The token rows, which all four waves read, still meet in LDS, but they
+// travel global -> registers -> LDS (ds_write_b128) instead of straight to LDS: a wave
+// requests its JT loads of 8 rows of stage s+3 during stage s, into the registers whose
+// previous content (stage s+1) it has just written to LDS. Two LDS buffers of 4 KiB per
+// 32-row block, written one stage before they are read. Half the LDS traffic of the version
+// above is gone (no weight rows written, no weight fragments read), the hand-over between
+// two stages waits for LDS only (this wave's writes of stage s+1 and reads of stage s, then
+// the workgroup barrier), and every global load has 1.75 to 2 stages to arrive.
+//
+// Loads straight to LDS are not used here on purpose: a load to registers that was still
+// outstanding when a younger load-to-LDS was issued did not deliver its data (the register
+// kept its old content; measured, deterministic), and the two kinds are not counted in order
+// with each other either. With one kind of load only, completion is in order and how many
+// younger loads may stay in flight at each wait is a constant of the schedule: every wave
+// issues the same loads in the same order. direct_wait() counts them from the list of what
+// a stage issues (which also covers the last stages, where loads of stages that do not exist
+// are left out):
+//   sub-step 0: weights (s+1, sub-step 3); sub-step 1: weights (s+2, sub-step 0), then the
+//   token rows of stage s+3; sub-step 2, 3: weights (s+2, sub-step 1, 2).
+// The loads in front of the loop are issued in the same order, as if by stages -2 and -1.
+constexpr int DIRECT_GROUPS = 5;
+constexpr int DIRECT_JT_MAX = 8;     // taller tiles do not leave the registers for it
+constexpr int DIRECT_MIN_STAGES = 4;
+// Loads that group g (in issue order) of a stage with r stages after it puts out.
+constexpr int direct_group(int jt, int r, int g) {
+  switch (g) {
+    case 0: return r >= 1 ? 2 : 0;
+    case 2: return r >= 3 ? jt : 0;
+    default: return r >= 2 ? 2 : 0;
+  }
+}
+// Loads issued after group g0 of the stage `back` stages before the present one (which has
+// r stages after it) and before group g1 of the present stage: those may still be in flight
+// when everything up to and including that group has to have landed.
+constexpr int direct_in_flight(int jt, int r, int back, int g0, int g1) {
+  int n = 0;
+  for (int b = back; b >= 0; --b) {
+    const int lo = b == back ? g0 + 1 : 0;
+    const int hi = b == 0 ? g1 : DIRECT_GROUPS;
+    for (int g = lo; g < hi; ++g) n += direct_group(jt, r + b, g);
+  }
+  return n;
+}
+// wait in front of sub-step w of a stage with r stages after it: its weight fragments and,
+// for sub-step 0, the token rows of the next stage, which that sub-step writes to LDS
+constexpr int direct_wait(int jt, int r, int w) {
+  switch (w) {
+    case 0: return direct_in_flight(jt, r, 2, 2, 0);
+    case 1: return direct_in_flight(jt, r, 2, 3, 1);
+    case 2: return direct_in_flight(jt, r, 2, 4, 3);
+    default: return direct_in_flight(jt, r, 1, 0, 4);
+  }
+}
+
+typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
+
+template <bool INIT>
+__device__ __forceinline__ void mma32v(const v4u_t& av, const uint4& b, f32x16& c) {
+  const v4u_t bv = {b.x, b.y, b.z, b.w};
+  if (INIT) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(av), "v"(bv));
+  } else {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
+  }
+}
+
+// 16 bytes per lane from base + off into the registers of `dst`; completion is tracked by
+// hand (wait_vm), so the compiler must not believe it knows when the value is there: the
+// operand is read-write, which keeps the value in one place from the load to its last use.
+__device__ __forceinline__ void load_fragment(v4u_t& dst, unsigned off, const unsigned char* base) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "+v"(dst) : "v"(off), "s"(base) : "memory");
+}
+// 16 bytes per lane from registers to LDS (byte address `lds_off`)
+__device__ __forceinline__ void store_fragment(unsigned lds_off, const v4u_t& src) {
+  asm volatile("ds_write_b128 %0, %1" : : "v"(lds_off), "v"(src) : "memory");
+}
+
+template <int JT>
+__device__ __forceinline__ void tile_gemm_direct(const TileOperands& op, int nstages, f32x16 (&acc)[2][JT_MAX],
+                                                 unsigned* pend, unsigned* queue, unsigned& next) {
+  static_assert(JT <= DIRECT_JT_MAX, "tile too tall for the register-staged pipeline");
+  constexpr int NS = 8;                           // slots per sub-step
+  constexpr int BAR = 2;                          // pairs of sub-step 3 in front of the hand-over
+  constexpr int AFTER = NS - BAR;
+  constexpr int STG = 32 * JT * ROWB;             // token rows of one stage
+  constexpr int RPS = (JT + AFTER - 1) / AFTER;   // reads of the next stage's first fragments per slot behind the hand-over
+  static_assert(2 * STG <= TILE_LDS_BYTES, "token stages exceed the tile's LDS");
+  const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6);
+  const int r32 = lane & 31, kq = lane >> 5;
+  const unsigned lds_addr = uni(static_cast<unsigned>(
+      reinterpret_cast<size_t>((FMOE_L3 unsigned char*)lds_raw)));
+
+  int fo[4];  // per-lane token fragment offsets of the four 16-k sub-steps
+#pragma unroll
+  for (int u = 0; u < 4; ++u) fo[u] = r32 * ROWB + (((2 * u + kq) ^ ((r32 >> 1) & 7)) << 4);
+  // weight fragment (sub-step u, 32-row block i) of stage s in the wave's packed slice:
+  // 8192*s + 4096*(u/2) + 2048*i + 512*(u%2), plus this lane's part
+  const unsigned aoff = static_cast<unsigned>(((r32 >> 4) << 10) + (kq << 8) + ((r32 & 15) << 4));
+  // where this lane's 16 bytes of the wave's token load q belong in a stage buffer: the
+  // eight rows of load q are one run of 1 KiB, lane l at 16*l
+  const unsigned wr_off = lds_addr + static_cast<unsigned>((wave * JT) * 1024 + lane * 16);
+
+  v4u_t as[2][4][2];   // weight fragments: [stage parity][sub-step][block]
+  v4u_t bs[2][JT];     // token rows on their way to LDS: [stage parity][load]
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) as[p][u][i] = v4u_t{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int q = 0; q < JT; ++q) bs[p][q] = v4u_t{0u, 0u, 0u, 0u};
+  }
+  uint4 bf[2][JT_MAX];
+
+  auto issue_a = [&](int s, int u, int i, v4u_t& dst) {
+    load_fragment(dst, aoff, op.wbase + static_cast<size_t>(s) * 8192 + ((u >> 1) * 4096 + i * 2048 + (u & 1) * 512));
+  };
+  auto issue_b = [&](int s, int q, v4u_t& dst) {  // q-th token load of this wave for stage s
+    load_fragment(dst, op.toff[q], op.tbase + static_cast<size_t>(s) * ROWB);
+  };
+  auto write_b = [&](int buf, int q, const v4u_t& src) { store_fragment(wr_off + buf * STG + q * 1024, src); };
+  auto read_b = [&](int buf, int u, int j) {
+    return *reinterpret_cast<const uint4*>(
+        __builtin_assume_aligned(lds_raw + buf * STG + fo[u] + j * (32 * ROWB), 16));
+  };
+  auto pair = [&](auto init_tag, const v4u_t (&a)[2], const uint4 (&b)[JT_MAX], int j) {
+    constexpr bool INIT = decltype(init_tag)::value;
+    if (j < JT) {
+      mma32v<INIT>(a[0], b[j], acc[0][j]);
+      mma32v<INIT>(a[1], b[j], acc[1][j]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- in front of the loop. First what stage 0 needs at once: its token rows, its weight
+  // fragments, and the token rows of stage 1 (which stage 0 writes to LDS).
+#pragma unroll
+  for (int q = 0; q < JT; ++q) issue_b(0, q, bs[0][q]);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) issue_a(0, 0, i, as[0][0][i]);
+#pragma unroll
+  for (int q = 0; q < JT; ++q) issue_b(1, q, bs[1][q]);
+#pragma unroll
+  for (int u = 1; u < 4; ++u)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) issue_a(0, u, i, as[0][u][i]);
+  // Everything requested so far has landed, and so have the stores of the previous task's
+  // epilogue (loads and stores do not complete in order with each other, so only a wait for
+  // all of them covers the stores): behind the workgroup barrier thread 0 may signal that
+  // task's completion, and draws the ticket of the task after this one.
+  wait_vm<0>();
+#pragma unroll
+  for (int q = 0; q < JT; ++q) write_b(0, q, bs[0][q]);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  if (threadIdx.x == 0) {
+    if (pend != nullptr) (void)add_relaxed(pend, 1u);
+    next = add_relaxed(queue, 1u);
+  }
+  // then what stage -1 would have issued
+#pragma unroll
+  for (int i = 0; i < 2; ++i) issue_a(1, 0, i, as[1][0][i]);
+#pragma unroll
+  for (int q = 0; q < JT; ++q) issue_b(2, q, bs[0][q]);
+#pragma unroll
+  for (int u = 1; u < 3; ++u)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) issue_a(1, u, i, as[1][u][i]);
+#pragma unroll
+  for (int j = 0; j < JT; ++j) bf[0][j] = read_b(0, 0, j);
+
+  // One stage. P: its parity (which weight registers it multiplies, which LDS buffer it
+  // reads). R: stages after it, 3 meaning 3 or more.
+  auto stage = [&](auto par_tag, auto rem_tag, auto first_tag, int s) {
+    constexpr int P = decltype(par_tag)::value;
+    constexpr int R = decltype(rem_tag)::value;
+    constexpr bool A2 = R >= 2, A13 = R >= 1, B3 = R >= 3, NEXT = R >= 1;
+    using No = std::false_type;
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      if (u == 0) wait_vm<direct_wait(JT, R, 0)>();
+      if (u == 1) wait_vm<direct_wait(JT, R, 1)>();
+      if (u == 2) wait_vm<direct_wait(JT, R, 2)>();
+      const uint4 (&cur)[JT_MAX] = bf[u & 1];
+      uint4 (&nxt)[JT_MAX] = bf[(u + 1) & 1];
+#pragma unroll
+      for (int j = 0; j < NS; ++j) {
+        if (u == 0) {
+          pair(first_tag, as[P][u], cur, j);
+        } else {
+          pair(No{}, as[P][u], cur, j);
+        }
+        if (u == 0) {
+          if (j < 2 && A13) issue_a(s + 1, 3, j, as[1 - P][3][j]);
+          if (j < JT && NEXT) write_b(1 - P, j, bs[1 - P][j]);   // token rows of stage s+1
+        } else if (u == 1) {
+          if (j == 0 && A2) {
+            issue_a(s + 2, 0, 0, as[P][0][0]);
+            issue_a(s + 2, 0, 1, as[P][0][1]);
+          }
+          if (j < JT && B3) issue_b(s + 3, j, bs[1 - P][j]);
+        } else if (j < 2 && A2) {
+          issue_a(s + 2, 1, j, as[P][1][j]);
+        }
+        if (j < JT) nxt[j] = read_b(P, u + 1, j);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    wait_vm<direct_wait(JT, R, 3)>();
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+      if (j == BAR) {
+        // this wave no longer reads this stage's buffer and has written its part of the next
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (NEXT) {
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+        }
+      }
+      pair(No{}, as[P][3], bf[1], j);
+      if (j < 2 && A2) issue_a(s + 2, 2, j, as[P][2][j]);
+      if (j >= BAR && NEXT) {
+#pragma unroll
+        for (int r = (j - BAR) * RPS; r < (j - BAR + 1) * RPS; ++r)
+          if (r < JT) bf[0][r] = read_b(1 - P, 0, r);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using R3 = std::integral_constant<int, 3>;
+  // nstages is even and at least 4; stages with 3 or more after them: nstages - 3 (odd)
+  stage(P0{}, R3{}, Yes{}, 0);
+  int s = 1;
+  for (; s + 3 < nstages; s += 2) {
+    stage(P1{}, R3{}, No{}, s);
+    stage(P0{}, R3{}, No{}, s + 1);
+  }
+  stage(P1{}, std::integral_constant<int, 2>{}, No{}, s);
+  stage(P0{}, std::integral_constant<int, 1>{}, No{}, s + 1);
+  stage(P1{}, std::integral_constant<int, 0>{}, No{}, s + 2);
+  // the compiler does not see matrix instructions in the assembly above: keep the wait states
+  // between the last of them and the first read of an accumulator
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  wait_vm<0>();
+  __syncthreads();  // the stages are free for the epilogue
+}
+
 // Weights in the packed layout (the streaming variant's: per wave task and 32-k step four
 // runs of 1 KiB, one per 16-row block, each [16-byte chunk 0..3][row 0..15]). This wave's 64
 // stage rows are exactly one packed task: gate/up task (expert, 32 h columns) = gate blocks
@@ -755,12 +1016,14 @@ __device__ __forceinline__ unsigned packed_run_offset(int q) {
 template <int JT, bool down>
 __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int rows, int nblk, unsigned* pend,
                                           unsigned* queue) {
-#ifdef FMOE_TRACE_PHASES
-  const long long ph0 = wall_clock64();
-#endif
   const int H = uni(p.H), I = uni(p.I), K = uni(p.K);
   const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
   constexpr int NTL = ntl_of(JT);
+  // packed weights and at least four stages: the deeper pipeline (tile_gemm_direct), where a
+  // wave brings JT token loads per stage instead of NTL
+  const bool direct = JT <= DIRECT_JT_MAX &&
+                      uni(((down ? p.ffn2_packed : p.ffn1_packed) != nullptr && (down ? I : H) >= DIRECT_MIN_STAGES * KS) ? 1 : 0) != 0;
+  const int tl_per_wave = direct ? JT : NTL;
   const int* perm = uni(p.perm) + row0;
   const int n0 = uni(nblk) * (down ? TN : G1_COLS);
   TileOperands op;
@@ -793,7 +1056,7 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
     }
 #pragma unroll
     for (int q = 0; q < NTL; ++q) {
-      const int row = stage_row(NTL, q);
+      const int row = stage_row(tl_per_wave, q);
       op.toff[q] = static_cast<unsigned>(min(row, rows - 1)) * static_cast<unsigned>(I * 2) + stage_chunk_bytes(row);
     }
   } else {
@@ -821,25 +1084,19 @@ __device__ __forceinline__ void tile_task(ParamsRef p, int expert, int row0, int
     }
 #pragma unroll
     for (int q = 0; q < NTL; ++q) {
-      const int row = stage_row(NTL, q);
+      const int row = stage_row(tl_per_wave, q);
       const int tok = ldc(&perm[min(row, rows - 1)]) / K;
       op.toff[q] = static_cast<unsigned>(tok) * static_cast<unsigned>(H * 2) + stage_chunk_bytes(row);
     }
   }
   f32x16 acc[2][JT_MAX];
-#ifdef FMOE_TRACE_PHASES
-  const long long ph1 = wall_clock64();
-  const long long pc1 = clock64();
-#endif
   unsigned next = 0u;
-  tile_gemm<JT>(op, nstages, acc, pend, queue, next);
-  if (threadIdx.x == 0) task_notes()[0] = next;  // the epilogue's barriers publish it
-#ifdef FMOE_TRACE_PHASES
-  if (threadIdx.x == 0) {
-    task_notes()[1] = static_cast<unsigned>(ph1 - ph0);
-    task_notes()[2] = static_cast<unsigned>(wall_clock64() - ph1) | (static_cast<unsigned>((clock64() - pc1) >> 6) << 16);
+  if (direct) {
+    if constexpr (JT <= DIRECT_JT_MAX) tile_gemm_direct<JT>(op, nstages, acc, pend, queue, next);
+  } else {
+    tile_gemm<JT>(op, nstages, acc, pend, queue, next);
   }
-#endif
+  if (threadIdx.x == 0) task_notes()[0] = next;  // the epilogue's barriers publish it
 
   const int r32 = lane & 31, kq = lane >> 5;
   unsigned char* slab = lds_raw;
@@ -961,10 +1218,115 @@ constexpr int TILED_LDS_BYTES =
 // combine: out[t] = sum over slots, in slot order, of w[t,slot] * y[t*K+slot]
 // (refFullMoe.h:35,62-65): y holds each slot's down-projection row rounded to bf16; weight
 // and sum are float, one fused multiply-add per slot, then one rounding to bf16.
-#ifndef FMOE_CMB_U
-#define FMOE_CMB_U 4
-#endif
-constexpr int CMB_U = FMOE_CMB_U;  // items a thread of the combine task has in flight
+//
+// One item = 8 columns of one token; a unit = the rows of up to 8 slots of one item (16
+// bytes each). A thread walks through its units with the loads of the next CMB_D - 1 units
+// in flight while it sums the present one: with one wave per SIMD nothing else covers the
+// summing, and a thread that loads everything and then sums everything leaves the memory
+// pipeline idle half of the time (4.4 TB/s; measured with four items loaded at once).
+constexpr int CMB_D = 3;  // units of a thread: one being summed, the others in flight
+constexpr int CMB_RUN = 8;  // units of one straight-line run (30B shape: one task)
+// Every thread of the task walks through the same number of units with unconditional loads
+// (a thread without an item of its own repeats the task's last one and stores nothing; slots
+// past K repeat slot K-1 and are not summed), so control flow is uniform and every wave has
+// the same loads in flight. The loads are issued from assembly and waited for by count
+// (left to itself the compiler waited for all but one unit's loads before every sum).
+// Stores are not counted: they may complete out of order with the loads, and leaving them
+// out of the count only makes a wait longer, never shorter.
+__device__ __forceinline__ void load_once(v4u_t& dst, unsigned off, const unsigned char* base) {
+  asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
+template <bool RESIDUAL>
+__device__ __forceinline__ void combine_units(const unsigned short* y, const unsigned short* residual,
+                                              unsigned short* out, const float* wts, const unsigned char* flag,
+                                              int t0, int nitems, int cpr, int H, int K) {
+  constexpr int LPU = RESIDUAL ? 9 : 8;  // loads per unit
+  const int tid = threadIdx.x;
+  const int nchunks = uni((K + 7) >> 3);  // units per item
+  const int nunits = uni(((nitems + T_THREADS - 1) / T_THREADS) * nchunks);
+  v4u_t v[CMB_D][8];
+  v4u_t rv[CMB_D];
+  // the task's rows of y and of the residual (uniform); a lane's offsets inside them fit 32 bits
+  const unsigned char* ybase = uni(reinterpret_cast<const unsigned char*>(y + static_cast<size_t>(t0) * K * H));
+  const unsigned char* rbase = uni(reinterpret_cast<const unsigned char*>(residual + static_cast<size_t>(t0) * H));
+  auto where = [&](int unit, int& tl, int& col, int& k0, bool& live) {
+    const int item = unit / nchunks;  // uniform
+    k0 = (unit - item * nchunks) << 3;
+    const int it = tid + item * T_THREADS;
+    live = it < nitems;
+    const int itc = min(it, nitems - 1);
+    tl = itc / cpr;
+    col = (itc - tl * cpr) << 3;
+  };
+  auto issue = [&](int unit, v4u_t (&dst)[8], v4u_t& rdst) {
+    int tl, col, k0;
+    bool live;
+    where(unit, tl, col, k0, live);
+    const unsigned yoff = static_cast<unsigned>((tl * K * H + col) * 2);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) load_once(dst[k], yoff, ybase + static_cast<size_t>(min(k0 + k, K - 1)) * H * 2);
+    if (RESIDUAL) load_once(rdst, static_cast<unsigned>((tl * H + col) * 2), rbase);
+  };
+  float s[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = 0.0f;
+  auto consume = [&](int unit, const v4u_t (&src)[8], const v4u_t& rsrc) {
+    int tl, col, k0;
+    bool live;
+    where(unit, tl, col, k0, live);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int kk = min(k0 + k, K - 1);
+      // a slot without an expert holds rows nobody wrote: they are not looked at
+      const bool use = k0 + k < K && flag[tl * K + kk] != 0;
+      const float w = wts[tl * K + kk];
+      float f[8];
+      unpack<BF16>(make_uint4(src[k].x, src[k].y, src[k].z, src[k].w), f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s[i] = use ? __fmaf_rn(f[i], w, s[i]) : s[i];
+    }
+    if (k0 + 8 >= K) {  // the item's last unit (uniform)
+      if (RESIDUAL) {  // output = input row + layer, the row added last
+        float f[8];
+        unpack<BF16>(make_uint4(rsrc.x, rsrc.y, rsrc.z, rsrc.w), f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s[i] += f[i];
+      }
+      if (live)
+        st16(out + static_cast<size_t>(t0 + tl) * H + col,
+             u32x4{pack_bf16(s[0], s[1]), pack_bf16(s[2], s[3]), pack_bf16(s[4], s[5]), pack_bf16(s[6], s[7])});
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s[i] = 0.0f;
+    }
+  };
+  // Units go in straight-line runs of CMB_RUN (no loop-carried registers: a value that is
+  // still on its way from memory must never be copied), the rest one by one.
+  auto run = [&](auto n_tag, int u0) {
+    constexpr int N = decltype(n_tag)::value;
+#pragma unroll
+    for (int d = 0; d + 1 < CMB_D && d < N; ++d) issue(u0 + d, v[d], rv[d]);
+#pragma unroll
+    for (int d = 0; d < N; ++d) {
+      if (d + CMB_D - 1 < N) {
+        issue(u0 + d + CMB_D - 1, v[(d + CMB_D - 1) % CMB_D], rv[(d + CMB_D - 1) % CMB_D]);
+        wait_vm<(CMB_D - 1) * LPU>();
+      } else if (d + 2 < N && CMB_D > 3) {
+        wait_vm<2 * LPU>();
+      } else if (d + 1 < N) {
+        wait_vm<LPU>();
+      } else {
+        wait_vm<0>();
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      consume(u0 + d, v[d % CMB_D], rv[d % CMB_D]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  int u0 = 0;
+  for (; u0 + CMB_RUN <= nunits; u0 += CMB_RUN) run(std::integral_constant<int, CMB_RUN>{}, u0);
+  for (; u0 < nunits; ++u0) run(std::integral_constant<int, 1>{}, u0);
+}
+
 __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
   ParamsRef p = uniform_params(pv);
   const int H = uni(p.H), K = uni(p.K), T = uni(p.T), E = uni(p.E), W = uni(p.W);
@@ -976,7 +1338,7 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
   unsigned long long* masks = uni(p.masks);
   const int tid = threadIdx.x;
   const int t0 = uni(blk) * CMB_TOK;
-  const int ntok = min(CMB_TOK, T - t0);
+  const int ntok = uni(min(CMB_TOK, T - t0));
   // which (token, slot) pairs of this task hold an expert, and their gate weights: one load each
   float* wts = reinterpret_cast<float*>(lds_raw);                      // [CMB_TOK * MAX_TOPK]
   unsigned char* flag = lds_raw + CMB_TOK * MAX_TOPK * sizeof(float);  // [CMB_TOK * MAX_TOPK]
@@ -985,64 +1347,11 @@ __device__ __noinline__ void tiled_combine_task(ParamsRef pv, int blk) {
     wts[tid] = ldc(&topk_w[static_cast<size_t>(t0) * K + tid]);
   }
   __syncthreads();
-  // one item = 8 columns of one token; a thread works on CMB_U items at a time, so that
-  // CMB_U*K row loads are in flight per lane (one CU alone needs about 64 KiB in flight for
-  // its share of the memory bandwidth)
   const int cpr = H >> 3;  // items per token
-  const int nitems = ntok * cpr;
-  for (int it0 = tid; it0 < nitems; it0 += CMB_U * T_THREADS) {
-    float s[CMB_U][8];
-    unsigned valid[CMB_U];
-    const unsigned short* yrow[CMB_U];
-    const float* wrow[CMB_U];
-    int tok[CMB_U], col[CMB_U];
-#pragma unroll
-    for (int u = 0; u < CMB_U; ++u) {
-      const int it = min(it0 + u * T_THREADS, nitems - 1);
-      const int tl = it / cpr;
-      wrow[u] = wts + tl * K;
-      col[u] = (it - tl * cpr) << 3;
-      tok[u] = t0 + tl;
-      valid[u] = 0u;
-      for (int k = 0; k < K; ++k) valid[u] |= static_cast<unsigned>(flag[tl * K + k]) << k;
-      yrow[u] = y + static_cast<size_t>(tok[u]) * K * H + col[u];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) s[u][i] = 0.0f;
-    }
-    for (int k0 = 0; k0 < K; k0 += 8) {
-      uint4 v[CMB_U][8];
-#pragma unroll
-      for (int u = 0; u < CMB_U; ++u)
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-          if (k0 + k < K) v[u][k] = ld16_once(yrow[u] + static_cast<size_t>(k0 + k) * H);
-#pragma unroll
-      for (int u = 0; u < CMB_U; ++u)
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-          if (k0 + k < K && ((valid[u] >> (k0 + k)) & 1u)) {
-            float f[8];
-            unpack<BF16>(v[u][k], f);
-            const float w = wrow[u][k0 + k];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s[u][i] = __fmaf_rn(f[i], w, s[u][i]);
-          }
-    }
-    if (residual != nullptr) {  // output = input row + layer, the row added last
-#pragma unroll
-      for (int u = 0; u < CMB_U; ++u) {
-        float f[8];
-        unpack<BF16>(ld16(residual + static_cast<size_t>(tok[u]) * H + col[u]), f);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) s[u][i] += f[i];
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < CMB_U; ++u)
-      if (it0 + u * T_THREADS < nitems)
-        st16(out + static_cast<size_t>(tok[u]) * H + col[u],
-             u32x4{pack_bf16(s[u][0], s[u][1]), pack_bf16(s[u][2], s[u][3]), pack_bf16(s[u][4], s[u][5]),
-                   pack_bf16(s[u][6], s[u][7])});
+  if (residual != nullptr) {
+    combine_units<true>(y, residual, out, wts, flag, t0, ntok * cpr, cpr, H, K);
+  } else {
+    combine_units<false>(y, residual, out, wts, flag, t0, ntok * cpr, cpr, H, K);
   }
   for (int tl = 0; tl < ntok; ++tl) {
     const int t = t0 + tl;
@@ -1108,13 +1417,8 @@ __global__ __launch_bounds__(T_THREADS) __attribute__((disable_tail_calls)) void
       st16(reinterpret_cast<char*>(r) + 16,
            u32x4{static_cast<unsigned>(t_fetch), static_cast<unsigned>(t_fetch >> 32),
                  static_cast<unsigned>(t_ready), static_cast<unsigned>(t_ready >> 32)});
-#ifdef FMOE_TRACE_PHASES
-      const unsigned x0 = task_notes()[1], x1 = task_notes()[2];
-#else
-      const unsigned x0 = 0u, x1 = 0u;
-#endif
       st16(reinterpret_cast<char*>(r) + 32,
-           u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), x0, x1});
+           u32x4{static_cast<unsigned>(t_end), static_cast<unsigned>(t_end >> 32), 0u, 0u});
     }
   };
 

@@ -163,6 +163,8 @@ def test_relaunch_across_batch_sizes(sched):
     (1100, 256, 8, 2, 128),     # ~275 rows per expert: tall tiles (a tail of <= 64 rows joins the full tile)
     (1180, 512, 4, 1, 256),     # ~295 rows per expert, top-1; some experts beyond 320 rows (tile + tail tile)
     (4100, 256, 200, 6, 128),   # more than one round of 16-token router tasks: 32-token tasks, two expert slabs, ragged last task
+    (900, 768, 8, 2, 384),      # twelve and six 64-k stages: the packed weights' deeper pipeline past its first and last stages
+    (2500, 512, 8, 1, 640),     # ~312 rows per expert: tiles of nine and ten 32-row blocks on three token buffers
 ])
 def test_tiled_variant_forced(shape):
     T, H, E, k, I = shape
