@@ -68,7 +68,14 @@ C_ABI = {
     "flashMoeTraceEnable": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "flashMoeTraceRead": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint,
                                          ctypes.c_void_p]),
+    "flashMoeReadDownRows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
+                                            ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                            ctypes.c_void_p]),
+    "flashMoeNoAllocStatus": (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint), ctypes.c_void_p]),
+    "flashMoeAbi": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_size_t)]),
+    "flashMoeSetDenseSmallBatch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
 }
+ABI_VERSION = 3
 # the C++-typed entry points of include/iMoeKernelLauncher.h (checked for presence only)
 CXX_ABI = ["CreateLauncher", "CreateLauncherEx", "DestroyLauncher", "GetDistributedUniqueId",
            "LauncherHandle"]
@@ -89,5 +96,13 @@ def load():
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
+        # a library built from another header revision would read the description wrongly
+        version, desc_bytes = ctypes.c_int(0), ctypes.c_size_t(0)
+        if lib.flashMoeAbi(ctypes.byref(version), ctypes.byref(desc_bytes)) != HIP_SUCCESS or \
+                version.value != ABI_VERSION or desc_bytes.value != ctypes.sizeof(LayerDesc):
+            raise RuntimeError("libflashMoe.so has interface revision %d with a %d-byte layer "
+                               "description; this binding is written for revision %d and %d bytes: "
+                               "rebuild the library" % (version.value, desc_bytes.value, ABI_VERSION,
+                                                        ctypes.sizeof(LayerDesc)))
         _lib = lib
     return _lib

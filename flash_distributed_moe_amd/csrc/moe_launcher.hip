@@ -294,7 +294,20 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
 
 extern "C" {
 
-const char* flashMoeVersion(void) { return "flashMoe-mi355x 0.1 (gfx950)"; }
+const char* flashMoeVersion(void) { return "flashMoe-mi355x 0.3 (gfx950)"; }
+
+int flashMoeAbi(int* version, size_t* desc_bytes) {
+  if (version == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null result pointer");
+  *version = FLASH_MOE_ABI_VERSION;
+  if (desc_bytes != nullptr) *desc_bytes = sizeof(FlashMoeLayerDesc);
+  return hipSuccess;
+}
+
+int flashMoeSetDenseSmallBatch(FlashMoeLauncher* l, int enable) {
+  (void)l;
+  (void)enable;
+  return hipSuccess;
+}
 
 int flashMoeWorkspaceBytes(const FlashMoeLayerDesc* desc, size_t* bytes) {
   const hipError_t v = validate(desc);
@@ -471,7 +484,10 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
 // code object and held until the process ends. In host code the array's name is
 // only a handle for hipGetSymbolAddress; the device address it yields, kept per
 // device in g_static, is what kernels, fills and copies are given.
-static __device__ __align__(256) unsigned char scratch[FLASH_MOE_NOALLOC_SCRATCH_BYTES];
+// Behind the workspace proper: one line whose first word collects the error bits of failed
+// launches (the clearing kernel leaves it alone; flashMoeNoAllocStatus reads and clears it).
+constexpr size_t kScratchErrorOffset = FLASH_MOE_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[FLASH_MOE_NOALLOC_SCRATCH_BYTES + 256];
 
 namespace {
 
@@ -505,6 +521,17 @@ hipError_t static_device(int device, const StaticDevice** out) {
       sd.ticks_per_ms = khz;
     FMOE_HIP_CHECK(fmoe::prepare_stream_kernel());
     FMOE_HIP_CHECK(fmoe::prepare_tiled_kernel());
+    // as in flashMoeCreate: every workgroup of a launch must be resident at once
+    int per_cu = 0;
+    FMOE_HIP_CHECK(fmoe::stream_kernel_occupancy(FLASH_MOE_BF16, &per_cu));
+    if (per_cu < 1) FMOE_FAIL(hipErrorLaunchOutOfResources, "the streaming kernel does not fit a CU");
+    FMOE_HIP_CHECK(fmoe::stream_kernel_occupancy(FLASH_MOE_F32, &per_cu));
+    if (per_cu < 1) FMOE_FAIL(hipErrorLaunchOutOfResources, "the streaming kernel does not fit a CU");
+    FMOE_HIP_CHECK(fmoe::tiled_kernel_occupancy(&per_cu));
+    if (per_cu < 1) FMOE_FAIL(hipErrorLaunchOutOfResources, "the tiled kernel does not fit a CU");
+    // the error word starts at zero (the array is zero-initialised with the code object,
+    // but a process may have failed launches behind it)
+    FMOE_HIP_CHECK(hipMemset(static_cast<unsigned char*>(ptr) + kScratchErrorOffset, 0, 256));
     sd.ptr = static_cast<unsigned char*>(ptr);
     sd.ready = true;
   }
@@ -566,6 +593,9 @@ int flashMoeLaunchNoAlloc(const FlashMoeLayerDesc* desc, const void* tokens, voi
   l.num_cus = sd->num_cus;
   l.ticks_per_ms = sd->ticks_per_ms;
   l.spin_limit = 2000 * sd->ticks_per_ms;
+  // where a failing launch's last worker leaves its error bits: device memory here, no
+  // pinned host word (that would be an allocation)
+  l.host_error_dev = reinterpret_cast<unsigned*>(sd->ptr + kScratchErrorOffset);
 
   // The array keeps what the last call (of any shape) left in it: counters, flags
   // and masks of this call's layout must start at zero. A kernel, not a memset,
@@ -583,6 +613,23 @@ int flashMoeLaunchNoAlloc(const FlashMoeLayerDesc* desc, const void* tokens, voi
   } else {
     FMOE_HIP_CHECK(fmoe::launch_stream_kernel(p, desc->dtype, p.n_groups, stream));
   }
+  return hipSuccess;
+}
+
+int flashMoeNoAllocStatus(unsigned* error_bits, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (error_bits == nullptr) FMOE_FAIL(hipErrorInvalidValue, "null result pointer");
+  int device = 0;
+  FMOE_HIP_CHECK(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) FMOE_FAIL(hipErrorInvalidDevice, "device %i", device);
+  const StaticDevice* sd = nullptr;
+  const hipError_t se = static_device(device, &sd);
+  if (se != hipSuccess) return se;
+  FMOE_HIP_CHECK(hipStreamSynchronize(stream));
+  unsigned bits = 0;
+  FMOE_HIP_CHECK(hipMemcpy(&bits, sd->ptr + kScratchErrorOffset, sizeof(bits), hipMemcpyDeviceToHost));
+  if (bits != 0u) FMOE_HIP_CHECK(hipMemset(sd->ptr + kScratchErrorOffset, 0, sizeof(bits)));
+  *error_bits = bits;
   return hipSuccess;
 }
 
@@ -632,6 +679,25 @@ int flashMoeReadIntermediate(FlashMoeLauncher* l, int tokens_num, void* h, void*
   const size_t esz = l->desc.dtype == FLASH_MOE_BF16 ? 2 : 4;
   const size_t bytes = esz * static_cast<size_t>(tokens_num) * l->desc.top_k * l->desc.intermediate;
   FMOE_HIP_CHECK(hipMemcpy(h, l->ws + l->layout.h, bytes, hipMemcpyDeviceToHost));
+  return hipSuccess;
+}
+
+int flashMoeReadDownRows(FlashMoeLauncher* l, int tokens_num, void* y, int* elem_dtype, int* weighted,
+                         void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (l == nullptr || y == nullptr || elem_dtype == nullptr || weighted == nullptr)
+    FMOE_FAIL(hipErrorInvalidValue, "null argument");
+  if (tokens_num < 0 || tokens_num > l->desc.max_tokens)
+    FMOE_FAIL(hipErrorInvalidValue, "tokens_num = %i", tokens_num);
+  FMOE_HIP_CHECK(hipStreamSynchronize(stream));
+  const bool tiled = sched_for(l->desc, tokens_num) == FLASH_MOE_SCHED_TILED;
+  const size_t rows = static_cast<size_t>(tokens_num) * l->desc.top_k;
+  const size_t bytes = rows * l->desc.hidden * (tiled ? 2 : 4);
+  const size_t kept = (l->layout.xn - l->layout.y);  // the region's size up to the next one
+  if (bytes > kept) FMOE_FAIL(hipErrorInvalidValue, "the workspace keeps fewer down-projection rows than %zu", rows);
+  *elem_dtype = tiled ? FLASH_MOE_BF16 : FLASH_MOE_F32;
+  *weighted = tiled ? 0 : 1;
+  FMOE_HIP_CHECK(hipMemcpy(y, l->ws + l->layout.y, bytes, hipMemcpyDeviceToHost));
   return hipSuccess;
 }
 

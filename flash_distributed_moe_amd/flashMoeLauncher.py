@@ -188,6 +188,23 @@ class MoeKernelLauncher:
             return (raw.astype(np.uint32) << 16).view(np.float32)
         return raw
 
+    def down_rows(self, tokens_num):
+        """(y, weighted): the down projection's rows of the last launch as float32
+        [tokens_num*k, H], row t*k+slot, and whether they already carry the slot's gate
+        weight (the streaming variant's do, the tiled variant's do not)."""
+        if self._h is None:
+            raise RuntimeError("Launcher was destroyed")
+        _, hidden, _, k = self._shape
+        raw = np.empty((tokens_num * k, hidden), np.float32)
+        dtype, weighted = ctypes.c_int(-1), ctypes.c_int(-1)
+        with torch.cuda.device(self._device):
+            _hip_check(self._lib.flashMoeReadDownRows(self._h, tokens_num, raw.ctypes.data, ctypes.byref(dtype),
+                                                      ctypes.byref(weighted), _stream()), "flashMoeReadDownRows")
+        if dtype.value == _lib.BF16:
+            bits = raw.view(np.uint16).reshape(-1)[:tokens_num * k * hidden]
+            raw = (bits.astype(np.uint32) << 16).view(np.float32).reshape(tokens_num * k, hidden)
+        return raw, bool(weighted.value)
+
     def status(self):
         """(error_bits, completed_launches) after waiting for the current stream."""
         err, n = ctypes.c_uint(), ctypes.c_uint()

@@ -138,6 +138,13 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
  * workspace is laid out for tokens_num alone, and with FLASH_MOE_SCHED_AUTO the
  * variant is the one flashMoeLaunch would take if its workspace fits, else the
  * streaming one.
+ * A failure on the device (a dependency wait that ran out, a row-tile table that
+ * overflowed) is not returned by any call of this entry point: the launch's output
+ * is all NaN, the array is usable again, and the error bits (as in flashMoeStatus)
+ * are added to a word that flashMoeNoAllocStatus reads and clears.
+ * Cost when unused: the array is part of the library's code object, so every
+ * process that loads the library holds FLASH_MOE_NOALLOC_SCRATCH_BYTES (+256) of
+ * device memory on each device it touches, whether or not it calls this.
  * hipErrorUnknown when tokens_num > desc->max_tokens or when that batch needs
  * more workspace than the array holds (bf16, top-8, 128 experts: 847 tokens of
  * the H2048/I768 shape with the streaming variant and 1447 with the tiled one,
@@ -150,6 +157,12 @@ int flashMoeLaunch(FlashMoeLauncher* l, const void* tokens, void* output, int to
 #define FLASH_MOE_NOALLOC_SCRATCH_BYTES (64u << 20)
 int flashMoeLaunchNoAlloc(const FlashMoeLayerDesc* desc, const void* tokens, void* output,
                           int tokens_num, void* stream);
+
+/* Waits for `stream`, then reports and clears the error bits that launches of
+ * flashMoeLaunchNoAlloc on the current device have raised since the last call
+ * (1 = a dependency wait timed out, 2 = tile table overflow; 0 = none). Not for
+ * use under graph capture (it copies one word to the host). */
+int flashMoeNoAllocStatus(unsigned* error_bits, void* stream);
 
 /* Frees the workspace; synchronises `stream`. */
 int flashMoeDestroy(FlashMoeLauncher* l, void* stream);
@@ -171,6 +184,22 @@ int flashMoeReadRouting(FlashMoeLauncher* l, int tokens_num, int* topk_idx, floa
  * reference's stage test does
  * (test/singleGPU/cpp/moe/internal/moeExpertFFN1Test.hip:58-106). */
 int flashMoeReadIntermediate(FlashMoeLauncher* l, int tokens_num, void* h, void* stream);
+
+/* After a launch of tokens_num tokens: waits for `stream`, then copies the down
+ * projection's rows, as the combine step reads them, to the host:
+ * y [tokens_num*top_k, H], row t*top_k+slot = h[row of (t, slot)] . W2[expert]^T.
+ * The two variants keep them differently, which *elem_dtype and *weighted report:
+ * the streaming variant float32, already multiplied by the slot's gate weight
+ * (FLASH_MOE_F32, 1), the tiled variant bfloat16, unweighted (FLASH_MOE_BF16, 0).
+ * `y` must hold 4 bytes per element either way. Rows of slots without an expert
+ * are undefined. hipErrorInvalidValue if the launcher's workspace keeps fewer rows
+ * than asked for (the streaming variant of an AUTO launcher that hands larger
+ * batches to the tiled one). No counterpart in the reference's library; it lets a
+ * test check the down projection and its scaling apart from the slot sum, as
+ * the reference's stage tests do
+ * (test/singleGPU/cpp/moe/internal/moeExpertsTests.hip:389-475). */
+int flashMoeReadDownRows(FlashMoeLauncher* l, int tokens_num, void* y, int* elem_dtype, int* weighted,
+                         void* stream);
 
 /* Device-side failures. A dependency wait inside the kernel is bounded (see
  * flashMoeSetWaitLimitMs); when one runs out, or the row-tile table overflows,
@@ -206,6 +235,22 @@ int flashMoeTraceRead(FlashMoeLauncher* l, void* records, unsigned max_records, 
 int flashMoeSchedFor(FlashMoeLauncher* l, int tokens_num);
 
 const char* flashMoeVersion(void);
+
+/* Binary interface revision, for bindings that were built against another header.
+ * History: 1 = first release; 2 = FlashMoeLayerDesc grew by norm_weight and norm_eps
+ * (16 bytes at the end; flashMoeCreate reads the whole struct, so a caller built
+ * against revision 1 must be rebuilt), flashMoeSetDenseSmallBatch became a no-op;
+ * 3 = flashMoeAbi, flashMoeReadDownRows, flashMoeNoAllocStatus added (symbol version
+ * LIBFLASHMOE_MI355X_0.3), nothing changed or removed. *desc_bytes (may be NULL)
+ * receives sizeof(FlashMoeLayerDesc) as the library was built: a binding compares it
+ * with its own before it passes a description. */
+#define FLASH_MOE_ABI_VERSION 3
+int flashMoeAbi(int* version, size_t* desc_bytes);
+
+/* Retained for binaries built against revision 1: the dense small-batch mode it
+ * switched measured slower at every batch size and no longer exists. Does nothing,
+ * returns hipSuccess. */
+int flashMoeSetDenseSmallBatch(FlashMoeLauncher* l, int enable);
 
 #ifdef __cplusplus
 }

@@ -18,6 +18,7 @@ class GpuCase:
     def __init__(self, cfg, seed=7907, sched=_lib.SCHED_AUTO, max_tokens=None, inputs=None,
                  pack_weights=False, prepacked=False, norm_weight=None, norm_eps=1e-6, residual=False):
         self.cfg, self.seed = cfg, seed
+        self.pack_weights, self.prepacked = pack_weights, prepacked
         self.norm_weight, self.norm_eps, self.residual = norm_weight, norm_eps, residual
         self.dev = torch.device("cuda:0")
         self.inp = inputs or synth.make_inputs_torch(cfg, seed, self.dev)

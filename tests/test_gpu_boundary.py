@@ -191,3 +191,45 @@ def test_gate_up_stage_alone(shape):
         print("  gate/up stage: %d rows checked" % len(r["perm"]), flush=True)
     finally:
         case.close()
+
+
+@pytest.mark.parametrize("shape", [
+    # T, H, E, k, I, dtype, sched
+    (24, 64, 4, 2, 32, "f32", 1),
+    (40, 128, 8, 2, 64, "bf16", 1),
+    (300, 256, 8, 2, 128, "bf16", 2),     # the tiled variant: bf16 rows, weight applied by the combine step
+    (700, 512, 4, 2, 256, "bf16", 2),     # the tiled variant on packed weights (register-staged pipeline)
+])
+def test_down_stage_alone(shape):
+    """The down projection and its scaling by themselves, as the reference tests its expert
+    stages apart from the sum over slots
+    (test/singleGPU/cpp/moe/internal/moeExpertsTests.hip:389-475): the rows the combine step
+    reads, copied back from the device, against the oracle's expert stage for that one
+    (token, slot) alone: with the slot's gate weight where the variant keeps weighted rows,
+    with weight 1 where it keeps them unweighted."""
+    T, H, E, k, I, dt, sched = shape
+    cfg = synth.MoeConfig("ffn2", T, H, E, k, I, dt)
+    case = GpuCase(cfg, seed=T + H, sched=sched, pack_weights=(H == 512))
+    try:
+        case.run()
+        r = case.launcher.routing(T)
+        y, weighted = case.launcher.down_rows(T)
+        assert weighted == (sched == 1)
+        hw = case.host_weights()
+        x = case.inp["tokens"].float().cpu().numpy()
+        one_idx = np.zeros((1, 1), np.int32)
+        checked = 0
+        for t in range(0, T, 1 if T <= 64 else 7):
+            for s in range(k):
+                e = int(r["topk_idx"][t, s])
+                w = np.full((1, 1), r["topk_w"][t, s] if weighted else 1.0, np.float32)
+                want = oracle.experts(x[t:t + 1], hw["ffn1"][e][None], hw["ffn2"][e][None], one_idx, w)[0]
+                got = y[t * k + s]
+                scale = max(float(np.abs(want).max()), 1e-12)
+                tol = 2e-5 if dt == "f32" else 1e-2
+                assert float(np.abs(got - want).max()) <= tol * scale, (t, s, e)
+                checked += 1
+        print("  down stage: %d rows checked, %s" % (checked, "weighted float rows" if weighted else "unweighted bf16 rows"),
+              flush=True)
+    finally:
+        case.close()
