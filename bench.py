@@ -36,16 +36,16 @@ BOUND = {
 
 # HBM bytes per launch as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch)
 # live in profiles/traffic.json, one entry per workload, each with the digest of the kernel
-# sources it was measured on. An entry whose digest differs from the tree's is stale and is
-# not reported (traffic: null). `bench.py --record-traffic FETCH_KIB WRITE_KIB` writes the entry
+# sources (device code) it was measured on. An entry whose digest differs from the tree's is
+# stale: `traffic` is null then and the old figure is shown as `traffic_stale`. `bench.py --record-traffic FETCH_KIB WRITE_KIB` writes the entry
 # of --config after a new pair of counter runs. Each counter is scaled by what it reads for a
 # plain copy of 1 GiB (bench.py --copy-calibration under the same counters): WRITE_SIZE 1.000,
 # FETCH_SIZE 0.500 (this chip reads HBM in 128-byte requests, which the counter's formula
 # prices at 64 bytes each).
 FETCH_SCALE = 0.5
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
-KERNEL_SOURCES = ["moe_stream_kernel.hip", "moe_tiled_kernel.hip", "moe_device.h", "moe_params.h",
-                  "moe_launcher.hip"]
+# device code only: the host launcher does not change what a kernel reads or writes
+KERNEL_SOURCES = ["moe_stream_kernel.hip", "moe_tiled_kernel.hip", "moe_device.h", "moe_params.h"]
 
 
 def kernel_sources_digest():
@@ -59,17 +59,18 @@ def kernel_sources_digest():
 
 
 def measured_traffic(workload, packed):
-    """Bytes per launch from profiles/traffic.json, or None if there is no entry for this
-    workload and weight layout measured on the present kernel sources."""
+    """(bytes per launch, stale) from profiles/traffic.json: bytes is None if there is no entry
+    for this workload and weight layout; stale says the entry was measured on other kernel
+    sources than the tree's."""
     try:
         with open(TRAFFIC_FILE) as f:
-            entry = json.load(f).get(workload)
+            entry = json.load(f).get(workload if packed else workload + ":row_major")
     except (OSError, ValueError):
-        return None
-    if not entry or entry.get("sources") != kernel_sources_digest() or \
-            bool(entry.get("packed_weights")) != bool(packed):
-        return None
-    return int((entry["fetch_kib"] / entry["fetch_scale"] + entry["write_kib"]) * 1024)
+        return None, False
+    if not entry or bool(entry.get("packed_weights")) != bool(packed):
+        return None, False
+    nbytes = int((entry["fetch_kib"] / entry["fetch_scale"] + entry["write_kib"]) * 1024)
+    return nbytes, entry.get("sources") != kernel_sources_digest()
 
 
 def record_traffic(workload, packed, fetch_kib, write_kib, kernel):
@@ -78,7 +79,7 @@ def record_traffic(workload, packed, fetch_kib, write_kib, kernel):
             table = json.load(f)
     except (OSError, ValueError):
         table = {}
-    table[workload] = {"kernel": kernel, "fetch_kib": fetch_kib, "write_kib": write_kib,
+    table[workload if packed else workload + ":row_major"] = {"kernel": kernel, "fetch_kib": fetch_kib, "write_kib": write_kib,
                        "fetch_scale": FETCH_SCALE, "packed_weights": bool(packed),
                        "sources": kernel_sources_digest()}
     with open(TRAFFIC_FILE, "w") as f:
@@ -149,7 +150,51 @@ def cpu_baseline(cfg, inp, seconds_budget=25.0):
     }
 
 
-def measure(name, seed, steps, warmup, sched, packed):
+def cold_cache_us(launcher, x, out, reps=20):
+    """Median duration of single launches that each follow a pass over a 1 GiB buffer, which
+    evicts the L2s and the 256 MB memory-side cache: the launch as a serving step meets it
+    when other layers have run in between."""
+    import torch
+
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device=x.device)
+    ts = []
+    for _ in range(reps):
+        flush.add_(1)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        launcher.launch(x, out)
+        b.record()
+        torch.cuda.synchronize()
+        ts.append(a.elapsed_time(b) * 1e3)
+    del flush
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def workgroup_balance(launcher, x, out, tokens, waves_per_group):
+    """Busy time per workgroup (= per CU: the launch puts one workgroup on each) of one traced
+    launch: sum of its tasks' durations as the kernel's own trace facility records them."""
+    import numpy as np
+    import torch
+
+    launcher.trace_enable(1 << 19)
+    launcher.launch(x, out)
+    torch.cuda.synchronize()
+    rec = launcher.trace_read()
+    launcher.trace_enable(0)
+    if len(rec) == 0:
+        return None
+    group = rec["worker"] // waves_per_group
+    busy = np.zeros(int(group.max()) + 1)
+    np.add.at(busy, group, (rec["t_end"] - rec["t_ready"]) / 100.0 / waves_per_group)
+    span = float(rec["t_end"].max() - rec["t_fetch"].min()) / 100.0
+    return {"workgroups": int(len(busy)), "busy_us_max": float(busy.max()), "busy_us_mean": float(busy.mean()),
+            "busy_us_min": float(busy.min()), "max_over_mean": float(busy.max() / busy.mean()),
+            "traced_span_us": span, "tasks": int(len(rec)), "tokens": int(tokens)}
+
+
+def measure(name, seed, steps, warmup, sched, packed, cold=False, balance=False):
     """K timed launches of workload `name`: whole-job wall time, the kernel's launch-to-launch
     duration from events on the launch stream, and where that puts it on its roofline."""
     import torch
@@ -202,7 +247,17 @@ def measure(name, seed, steps, warmup, sched, packed):
         sys.exit("bench.py: device error bits %d" % err)
     routing = launcher.routing(cfg.T)
     active = int((routing["counts"] > 0).sum())
-    kernel = "moe_stream_kernel" if launcher.sched_for(cfg.T) == 1 else "moe_tiled_kernel"
+    tiled = launcher.sched_for(cfg.T) != 1
+    kernel = "moe_tiled_kernel" if tiled else "moe_stream_kernel"
+    extra = {}
+    if cold:
+        extra["cold_cache_us"] = cold_cache_us(launcher, x, out)
+    if balance:
+        extra["per_cu_busy"] = workgroup_balance(launcher, x, out, cfg.T, 1 if tiled else 8)
+        counts = routing["counts"]
+        extra["rows_per_expert"] = {"max": int(counts.max()), "mean": float(counts.mean()),
+                                    "share_of_4_largest": float(sorted(counts)[-4:] and
+                                                                sum(sorted(counts)[-4:]) / max(1, counts.sum()))}
     launcher.destroy()
 
     bound = BOUND.get(cfg.name, "hbm")
@@ -215,16 +270,20 @@ def measure(name, seed, steps, warmup, sched, packed):
     else:
         achieved = aflops / (kernel_ms_avg * 1e-3) / 1e12
         peak, unit = mfma_peak, "TFLOP/s"
+    traffic, stale = measured_traffic(cfg.name, packed)
     roofline = {
         "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
         "frac": achieved / peak,
-        "traffic": measured_traffic(cfg.name, packed),
+        "traffic": None if stale else traffic,
         "kernel": kernel,
         "kernel_us_avg": kernel_ms_avg * 1e3, "kernel_us_median": kernel_ms_med * 1e3,
         "algorithmic_bytes": abytes, "algorithmic_flops": aflops, "active_experts": active,
         "hbm_frac": abytes / (kernel_ms_avg * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "mfma_frac": aflops / (kernel_ms_avg * 1e-3) / 1e12 / mfma_peak,
     }
+    if stale:
+        roofline["traffic_stale"] = traffic   # measured on other kernel sources than the tree's
+    roofline.update(extra)
     config = {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E,
               "top_k": cfg.k, "intermediate": cfg.I, "hot_experts": cfg.hot,
               "seed": seed, "packed_weight_copy": False,
@@ -245,7 +304,7 @@ def main():
     ap.add_argument("--no-pack-weights", action="store_true",
                     help="read the caller's row-major weight tensors instead of weights packed in place")
     ap.add_argument("--no-extra-records", action="store_true",
-                    help="only the one workload: no prefill and no caller's-layout sub-record")
+                    help="only the one workload: none of the sub-records of the other configurations")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy 1 GiB device to device five times: the known traffic the "
                          "rocprofv3 byte counters are scaled by")
@@ -264,7 +323,7 @@ def main():
         kernel = "moe_tiled_kernel" if BOUND.get(args.config) == "mfma" or "4096" in args.config \
             else "moe_stream_kernel"
         record_traffic(args.config, packed, args.record_traffic[0], args.record_traffic[1], kernel)
-        print(json.dumps({args.config: measured_traffic(args.config, packed)}))
+        print(json.dumps({args.config: measured_traffic(args.config, packed)[0]}))
         return
 
     import torch
@@ -309,8 +368,9 @@ def main():
         print(json.dumps({"gemm_calibration": out}))
         return
 
+    headline = args.config == "qwen3_30b_decode"
     cfg, inp, ms_per_step, roofline, config = measure(args.config, args.seed, args.steps,
-                                                      args.warmup, args.sched, packed)
+                                                      args.warmup, args.sched, packed, cold=headline)
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(cfg, inp)
@@ -334,19 +394,32 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
-    if not args.no_extra_records and args.config == "qwen3_30b_decode":
-        # the other headline workload (8192-token prefill, bound by the matrix cores) and the
-        # decode batch on the caller's weight layout (no packed copy), same fields
-        def sub(name, steps, warmup, packed_):
-            c, _, ms, roof, conf = measure(name, args.seed, steps, warmup, args.sched, packed_)
+    if not args.no_extra_records and headline:
+        # The other configurations the reference's numbers are asked for on, same fields each:
+        # the 8192-token prefill (bound by the matrix cores), the decode batch on the caller's
+        # row-major weights, the 235B shape at 256 and 4096 tokens (both roofline fractions are
+        # in every record: hbm_frac, mfma_frac) and the imbalance stress with the busy time per
+        # CU. Each is timed over at least 50 launches, so that ms_per_step is the kernel's
+        # time and not the cost of the final synchronisation.
+        import torch
+
+        def sub(name, packed_, balance=False):
+            steps, warmup = max(50, args.steps), max(5, args.warmup)
+            c, i_, ms, roof, conf = measure(name, args.seed, steps, warmup, args.sched, packed_,
+                                            balance=balance)
+            del i_
+            torch.cuda.empty_cache()
             return {"value": c.T / (ms * 1e-3), "unit": "tokens/s", "steps": steps, "warmup": warmup,
                     "ms_per_step": ms, "us_per_layer": ms * 1e3, "dtype": c.dtype, "config": conf,
                     "roofline": roof}
 
-        line["prefill"] = sub("qwen3_30b_prefill", max(10, args.steps // 4), max(3, args.warmup // 4),
-                              packed)
+        torch.cuda.empty_cache()
+        line["prefill"] = sub("qwen3_30b_prefill", packed)
         if packed:
-            line["caller_layout"] = sub("qwen3_30b_decode", args.steps, args.warmup, False)
+            line["caller_layout"] = sub("qwen3_30b_decode", False)
+        line["c4_t256"] = sub("qwen3_235b_t256", packed)
+        line["c4_t4096"] = sub("qwen3_235b_t4096", packed)
+        line["imbalance"] = sub("qwen3_30b_imbalance", packed, balance=True)
     print(json.dumps(line))
 
 

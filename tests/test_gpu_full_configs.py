@@ -31,7 +31,7 @@ HOST_THREADS = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREA
 _first_output = {}   # (config, T) -> output of the first variant run: later variants must match it
 
 
-def run_full(name, T=None, pack_weights=False, same_bits_as_first=False):
+def run_full(name, T=None, pack_weights=False, same_bits_as_first=False, fresh_relaunch=False):
     cfg = synth.CONFIGS[name]
     if T is not None:
         cfg = cfg.replace(T=T)
@@ -55,15 +55,56 @@ def run_full(name, T=None, pack_weights=False, same_bits_as_first=False):
             _first_output[key] = out.cpu()
         out2 = case.run(inplace=True)
         assert torch.equal(out, out2)                 # deterministic; aliasing-safe
+        if fresh_relaunch:
+            relaunch_with_fresh_tokens(case)
         return r
     finally:
         case.close()
 
 
+def relaunch_with_fresh_tokens(case):
+    """The launcher that has just run the checked batch runs two more batches of the same
+    size with other token contents, one eagerly and one as a replay of a captured graph, and
+    each must equal bit for bit what a launcher that has never run anything returns for those
+    tokens. The kernels' scratch rows (h, y, routing tables) are written through and read
+    back with ordinary cached loads by other workers at full occupancy: a line left over from
+    the previous launch would hold the previous batch's values and show here (the
+    reference's own check of that kind is
+    test/singleGPU/cpp/taskSystem/saxpyCoherenceTest.hip:113-143)."""
+    cfg = case.cfg
+    dt = torch.bfloat16 if cfg.dtype == "bf16" else torch.float32
+    fresh = [synth.normal_torch(s, synth.STREAM_TOKENS, (cfg.T, cfg.H), 1.0, dt, case.dev) for s in (4242, 777)]
+    assert not torch.equal(fresh[0], case.inp["tokens"])
+    other = GpuCase(cfg, inputs=case.inp, pack_weights=case.pack_weights)
+    try:
+        want = [other.run(tokens=f).clone() for f in fresh]
+    finally:
+        other.close()
+    got = case.run(tokens=fresh[0])
+    assert torch.equal(got, want[0]), "eager relaunch with fresh tokens differs from a fresh launcher"
+    # captured graph: warm-up on a side stream, capture one launch, replay it on the second batch
+    static_x, static_out = fresh[0].clone(), torch.empty_like(fresh[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        case.launcher.launch(static_x, static_out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        case.launcher.launch(static_x, static_out)
+    static_x.copy_(fresh[1])
+    g.replay()
+    torch.cuda.synchronize()
+    assert case.launcher.status()[0] == 0
+    assert torch.equal(static_out, want[1]), "graph replay with fresh tokens differs from a fresh launcher"
+    print("  relaunch (eager, then a graph replay) with fresh tokens: bit-equal to a fresh launcher", flush=True)
+
+
 @pytest.mark.parametrize("pack_weights", [False, True])
 def test_qwen3_30b_prefill(pack_weights):
     # the tiled variant reads the caller's layout either way
-    run_full("qwen3_30b_prefill", pack_weights=pack_weights, same_bits_as_first=True)
+    run_full("qwen3_30b_prefill", pack_weights=pack_weights, same_bits_as_first=True, fresh_relaunch=True)
 
 
 @pytest.mark.parametrize("pack_weights", [False, True])
@@ -73,11 +114,11 @@ def test_qwen3_235b_t256(pack_weights):
 
 
 def test_qwen3_235b_t4096():
-    run_full("qwen3_235b_t4096")
+    run_full("qwen3_235b_t4096", fresh_relaunch=True)
 
 
 def test_qwen3_30b_imbalance():
-    r = run_full("qwen3_30b_imbalance")
+    r = run_full("qwen3_30b_imbalance", fresh_relaunch=True)
     hot = synth.hot_experts(7907, 128, 4)
     share = r["counts"][hot].sum() / r["counts"].sum()
     print("  hot experts", hot, "share %.3f" % share, flush=True)
