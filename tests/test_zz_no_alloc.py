@@ -147,3 +147,42 @@ def test_no_alloc_rejects_what_does_not_fit(capfd):
     assert lib.flashMoeLaunchNoAlloc(ctypes.byref(d), x.data_ptr(), out.data_ptr(), 9, None) == _lib.HIP_ERROR_UNKNOWN
     d.flags = _lib.FLAG_PACK_WEIGHTS
     assert lib.flashMoeLaunchNoAlloc(ctypes.byref(d), x.data_ptr(), out.data_ptr(), 8, None) == _lib.HIP_ERROR_INVALID_VALUE
+
+
+def test_no_alloc_status_and_graph_capture():
+    """After a warm-up call (which looks up the static array's address) the call can be
+    recorded into a HIP graph: it allocates nothing and enqueues kernels only. Every replay
+    gets fresh tokens and must equal an eager launcher's result; flashMoeNoAllocStatus
+    reports no device error after them."""
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    for T, sched in ((40, _lib.SCHED_STREAM), (600, _lib.SCHED_TILED)):
+        cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=T, name="graph%d" % T)
+        inp = synth.make_inputs_torch(cfg, 7907, dev)
+        d = layer_desc(cfg, inp, T, sched)
+        static_x = inp["tokens"].clone()
+        static_out = torch.empty_like(static_x)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):   # warm-up outside the capture
+            rc = lib.flashMoeLaunchNoAlloc(ctypes.byref(d), static_x.data_ptr(), static_out.data_ptr(), T,
+                                           ctypes.c_void_p(side.cuda_stream))
+            assert rc == _lib.HIP_SUCCESS
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            rc = lib.flashMoeLaunchNoAlloc(ctypes.byref(d), static_x.data_ptr(), static_out.data_ptr(), T,
+                                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+            assert rc == _lib.HIP_SUCCESS
+        for rep in range(3):
+            fresh = synth.normal_torch(500 + rep, synth.STREAM_TOKENS, (T, cfg.H), 1.0, torch.bfloat16, dev)
+            static_x.copy_(fresh)
+            g.replay()
+            torch.cuda.synchronize()
+            want = with_launcher(cfg, inp, fresh, sched)   # eager work between the replays
+            assert torch.equal(static_out, want), "replay %d of the recorded no-alloc call differs" % rep
+        bits = ctypes.c_uint(99)
+        assert lib.flashMoeNoAllocStatus(ctypes.byref(bits), None) == _lib.HIP_SUCCESS
+        assert bits.value == 0
+        print("  no-alloc call recorded and replayed three times, T=%d sched=%d" % (T, sched), flush=True)
