@@ -58,29 +58,41 @@ def kernel_sources_digest():
     return h.hexdigest()[:16]
 
 
-def measured_traffic(workload, packed):
+WEIGHT_MODES = {
+    "in_place": "packed in place by the caller (flashMoePackWeightsInPlace), no second copy",
+    "default": "as a caller written against the reference gets them: row-major tensors handed to "
+               "create() with no flags, of which the launcher keeps a packed copy (+3*E*H*I elements)",
+    "row_major": "caller's row-major tensors read in place (create(..., flags=0))",
+}
+
+
+def traffic_key(workload, weights):
+    return workload if weights == "in_place" else workload + ":" + weights
+
+
+def measured_traffic(workload, weights):
     """(bytes per launch, stale) from profiles/traffic.json: bytes is None if there is no entry
     for this workload and weight layout; stale says the entry was measured on other kernel
     sources than the tree's."""
     try:
         with open(TRAFFIC_FILE) as f:
-            entry = json.load(f).get(workload if packed else workload + ":row_major")
+            entry = json.load(f).get(traffic_key(workload, weights))
     except (OSError, ValueError):
         return None, False
-    if not entry or bool(entry.get("packed_weights")) != bool(packed):
+    if not entry:
         return None, False
     nbytes = int((entry["fetch_kib"] / entry["fetch_scale"] + entry["write_kib"]) * 1024)
     return nbytes, entry.get("sources") != kernel_sources_digest()
 
 
-def record_traffic(workload, packed, fetch_kib, write_kib, kernel):
+def record_traffic(workload, weights, fetch_kib, write_kib, kernel):
     try:
         with open(TRAFFIC_FILE) as f:
             table = json.load(f)
     except (OSError, ValueError):
         table = {}
-    table[workload if packed else workload + ":row_major"] = {"kernel": kernel, "fetch_kib": fetch_kib, "write_kib": write_kib,
-                       "fetch_scale": FETCH_SCALE, "packed_weights": bool(packed),
+    table[traffic_key(workload, weights)] = {"kernel": kernel, "fetch_kib": fetch_kib, "write_kib": write_kib,
+                       "fetch_scale": FETCH_SCALE, "weights": weights,
                        "sources": kernel_sources_digest()}
     with open(TRAFFIC_FILE, "w") as f:
         json.dump(table, f, indent=1, sort_keys=True)
@@ -194,7 +206,7 @@ def workgroup_balance(launcher, x, out, tokens, waves_per_group):
             "traced_span_us": span, "tasks": int(len(rec)), "tokens": int(tokens)}
 
 
-def measure(name, seed, steps, warmup, sched, packed, cold=False, balance=False):
+def measure(name, seed, steps, warmup, sched, weights, cold=False, balance=False):
     """K timed launches of workload `name`: whole-job wall time, the kernel's launch-to-launch
     duration from events on the launch stream, and where that puts it on its roofline."""
     import torch
@@ -209,14 +221,15 @@ def measure(name, seed, steps, warmup, sched, packed, cold=False, balance=False)
     out = torch.empty_like(x)
     launcher = MoeKernelLauncher()
     ffn1, ffn2 = inp["ffn1"], inp["ffn2"]
-    if packed:
+    if weights == "in_place":
         # the layout the kernels read fastest, made where the tensors lie: the launcher keeps
         # no copy of the weights (the row-major originals stay in `inp` for the CPU baseline)
         ffn1, ffn2 = ffn1.clone(), ffn2.clone()
         MoeKernelLauncher.pack_weights_in_place(ffn1, ffn2)
     launcher.create(inp["gate"], ffn1, ffn2, cfg.T,
                     launcher.getDistributedUniqueId(empty=True), 0, 1, top_k=cfg.k,
-                    router_bias=inp["bias"], sched=sched, prepacked=packed)
+                    router_bias=inp["bias"], sched=sched, prepacked=weights == "in_place",
+                    pack_weights={"in_place": False, "default": None, "row_major": False}[weights])
     for _ in range(warmup):
         launcher.launch(x, out)
     torch.cuda.synchronize()
@@ -270,7 +283,7 @@ def measure(name, seed, steps, warmup, sched, packed, cold=False, balance=False)
     else:
         achieved = aflops / (kernel_ms_avg * 1e-3) / 1e12
         peak, unit = mfma_peak, "TFLOP/s"
-    traffic, stale = measured_traffic(cfg.name, packed)
+    traffic, stale = measured_traffic(cfg.name, weights)
     roofline = {
         "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
         "frac": achieved / peak,
@@ -286,9 +299,7 @@ def measure(name, seed, steps, warmup, sched, packed, cold=False, balance=False)
     roofline.update(extra)
     config = {"workload": cfg.name, "tokens": cfg.T, "hidden": cfg.H, "experts": cfg.E,
               "top_k": cfg.k, "intermediate": cfg.I, "hot_experts": cfg.hot,
-              "seed": seed, "packed_weight_copy": False,
-              "weights": "packed in place by the caller (flashMoePackWeightsInPlace), no second copy"
-                         if packed else "caller's row-major tensors"}
+              "seed": seed, "packed_weight_copy": weights == "default", "weights": WEIGHT_MODES[weights]}
     return cfg, inp, ms_per_step, roofline, config
 
 
@@ -301,8 +312,10 @@ def main():
     ap.add_argument("--seed", type=int, default=7907)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sched", type=int, default=0)
-    ap.add_argument("--no-pack-weights", action="store_true",
-                    help="read the caller's row-major weight tensors instead of weights packed in place")
+    ap.add_argument("--weights", default="in_place", choices=sorted(WEIGHT_MODES),
+                    help="in_place: weights packed in place by the caller (the headline); default: "
+                         "row-major tensors given to create() with no flags (the launcher keeps a "
+                         "packed copy); row_major: read in place")
     ap.add_argument("--no-extra-records", action="store_true",
                     help="only the one workload: none of the sub-records of the other configurations")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -318,7 +331,7 @@ def main():
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs the MoE layer on ONE GPU (no collectives, no "
                  "multi-GPU path); run with --gpus 1")
-    packed = not args.no_pack_weights
+    packed = args.weights
     if args.record_traffic:
         kernel = "moe_tiled_kernel" if BOUND.get(args.config) == "mfma" or "4096" in args.config \
             else "moe_stream_kernel"
@@ -396,8 +409,10 @@ def main():
     }
     if not args.no_extra_records and headline:
         # The other configurations the reference's numbers are asked for on, same fields each:
-        # the 8192-token prefill (bound by the matrix cores), the decode batch on the caller's
-        # row-major weights, the 235B shape at 256 and 4096 tokens (both roofline fractions are
+        # the 8192-token prefill (bound by the matrix cores), the decode batch as a caller written
+        # against the reference gets it (caller_layout: row-major tensors, create() without flags,
+        # the launcher's packed copy) and on the row-major tensors read in place
+        # (row_major_weights), the 235B shape at 256 and 4096 tokens (both roofline fractions are
         # in every record: hbm_frac, mfma_frac) and the imbalance stress with the busy time per
         # CU. Each is timed over at least 50 launches, so that ms_per_step is the kernel's
         # time and not the cost of the final synchronisation.
@@ -415,8 +430,8 @@ def main():
 
         torch.cuda.empty_cache()
         line["prefill"] = sub("qwen3_30b_prefill", packed)
-        if packed:
-            line["caller_layout"] = sub("qwen3_30b_decode", False)
+        line["caller_layout"] = sub("qwen3_30b_decode", "default")
+        line["row_major_weights"] = sub("qwen3_30b_decode", "row_major")
         line["c4_t256"] = sub("qwen3_235b_t256", packed)
         line["c4_t4096"] = sub("qwen3_235b_t4096", packed)
         line["imbalance"] = sub("qwen3_30b_imbalance", packed, balance=True)

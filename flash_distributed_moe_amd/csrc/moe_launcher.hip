@@ -157,12 +157,13 @@ hipError_t validate(const FlashMoeLayerDesc* d) {
 }
 
 // The tiled variant needs bf16, tile-aligned shapes and token rows it can
-// address with 32-bit byte offsets. AUTO takes it once an expert sees about 24
-// rows on average when the packed weight copy exists (30B shape, us, streaming /
-// tiled: T=320 283 / 282, T=384 292 / 284, T=512 333 / 289; 235B shape: T=384
-// 920 / 945, T=512 1025 / 960), and from about 3 rows when the weights are read
-// in the caller's row-major layout, which the streaming variant reads poorly
-// (30B: T=32 272 / 270, T=48 296 / 283, T=64 312 / 291, T=128 363 / 297).
+// address with 32-bit byte offsets. AUTO takes it once an expert sees about 22
+// rows on average when the weights are packed (30B shape, us, streaming / tiled:
+// T=256 288 / 299, T=320 298 / 299, T=384 306 / 301, T=512 340 / 304; 235B shape:
+// T=256 925 / 952, T=384 985 / 966, T=512 1064 / 977), and from about 14 rows on
+// the caller's row-major weights, which the streaming variant reads half a
+// cache line at a time (30B: T=64 272 / 315, T=128 287 / 315, T=192 309 / 316,
+// T=256 319 / 318, T=384 359 / 322; 235B: T=128 961 / 973, T=256 1036 / 996).
 bool tiled_eligible(const FlashMoeLayerDesc& d, int tokens_num) {
   return d.dtype == FLASH_MOE_BF16 && d.hidden % 256 == 0 && d.intermediate % 128 == 0 &&
          tokens_num <= fmoe::tiled_max_tokens() &&
@@ -175,7 +176,7 @@ int sched_for(const FlashMoeLayerDesc& d, int tokens_num) {
   if (d.sched == FLASH_MOE_SCHED_TILED) return FLASH_MOE_SCHED_TILED;
   const long long rows = static_cast<long long>(tokens_num) * d.top_k;
   const bool packed = (d.flags & (FLASH_MOE_FLAG_PACK_WEIGHTS | FLASH_MOE_FLAG_WEIGHTS_PREPACKED)) != 0;
-  return rows >= (packed ? 24ll : 3ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
+  return rows >= (packed ? 22ll : 14ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
 }
 
 // Whether any batch size up to max_tokens may run the tiled variant.
@@ -427,6 +428,17 @@ int flashMoeCreate(FlashMoeLauncher** out, const FlashMoeLayerDesc* desc, void* 
     return fail(e);
   if ((e = hipMemsetAsync(l->ws, 0, l->layout.zero_bytes, stream)) != hipSuccess) return fail(e);
   if (desc->flags & FLASH_MOE_FLAG_PACK_WEIGHTS) {
+    static bool announced = false;  // once per process: the cost must not go unseen
+    if (!announced) {
+      announced = true;
+      const double mib = static_cast<double>(l->layout.pack2 - l->layout.pack1 +
+                                             (l->layout.total - l->layout.pack2)) / (1024.0 * 1024.0);
+      // (a notice, not an error: to stderr, so that a program's own stdout stays its own)
+      fprintf(stderr,
+              "[MOE] launcher keeps a packed copy of the expert weights: +%.0f MiB of device memory per "
+              "launcher (FLASH_MOE_FLAG_PACK_WEIGHTS; without the flag the row-major tensors are read in "
+              "place, and flashMoePackWeightsInPlace needs no copy at all)\n", mib);
+    }
     if ((e = static_cast<hipError_t>(flashMoeRefreshWeights(l, stream))) != hipSuccess)
       return fail(e);
   }
@@ -822,6 +834,10 @@ hipError_t CreateLauncher(moe::IMoeKernelLauncher** launcher, const void* gateWe
   d.dtype = FLASH_MOE_F32;
   d.max_tokens = maxTokens;
   d.sched = FLASH_MOE_SCHED_AUTO;
+  // A caller of this entry point cannot say how its weights are to be read, so it gets the
+  // fast way: a packed copy in the workspace (announced by flashMoeCreate). CreateLauncherEx
+  // with flags = 0 reads the row-major tensors in place.
+  d.flags = FLASH_MOE_FLAG_PACK_WEIGHTS;
   d.gate_weights = gateWeights;
   d.ffn1_weights = ffn1ExpertWeights;
   d.ffn2_weights = ffn2ExpertWeights;

@@ -595,7 +595,27 @@ __device__ __forceinline__ bool wait_flag(ParamsRef p, int which, unsigned* lds_
 // the MFMAs; the other waves of the CU keep HBM busy meanwhile. `pre` runs once
 // after the first round's weight loads are in flight and before any B row is
 // touched (the down projection waits for its h rows there).
-template <typename DT, int NA, int RB, int U, bool COH_B, typename Pre>
+//
+// transpose_a (the caller's row-major weights): a fragment wants lane l to hold row l % 16,
+// 16-byte chunk l / 16 of a 64-byte row segment, which read that way makes every lane of a
+// load touch a line of its own.
+// So lane l loads chunk l % 4 of row l / 4 instead, four neighbouring lanes one contiguous
+// 64-byte segment, and the fragment is put right in registers afterwards: lane l takes the
+// four dwords of lane 4 * (l % 16) + l / 16 (ds_bpermute_b32: the LDS crossbar, no LDS memory).
+__device__ __forceinline__ uint4 fragment_from_row_order(const uint4& v, int pull_from) {
+  uint4 r;
+  r.x = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(pull_from, static_cast<int>(v.x)));
+  r.y = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(pull_from, static_cast<int>(v.y)));
+  r.z = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(pull_from, static_cast<int>(v.z)));
+  r.w = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(pull_from, static_cast<int>(v.w)));
+  return r;
+}
+// row and 16-byte chunk (of the 64-byte segment of one k-step) that this lane loads of a
+// 16-row weight block in the caller's row-major layout
+__device__ __forceinline__ int row_order_row() { return lane_id() >> 2; }
+__device__ __forceinline__ int row_order_chunk() { return lane_id() & 3; }
+
+template <typename DT, int NA, int RB, int U, bool COH_B, bool transpose_a, typename Pre>
 __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[NA],
                                            const typename DT::elem* const (&bp)[RB], int ksteps,
                                            int astep, f32x4 (&acc)[NA][RB], Pre pre,
@@ -619,7 +639,13 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int i = 0; i < NA; ++i) a[u][i] = ld16_once(ap[i] + static_cast<size_t>(s + u) * astep);
+      for (int i = 0; i < NA; ++i) {
+        // row-major rows are read half a line at a time: the other half comes with the next
+        // k-step and must find the line still cached, so these loads are ordinary ones (with
+        // the non-temporal hint the second half was fetched again: 64 tokens 300 -> 273 us)
+        a[u][i] = transpose_a ? ld16(ap[i] + static_cast<size_t>(s + u) * astep)
+                              : ld16_once(ap[i] + static_cast<size_t>(s + u) * astep);
+      }
   };
   auto load_b = [&](int s) {
 #pragma unroll
@@ -630,7 +656,14 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
         b[u][r] = ld_b(q);
       }
   };
+  const int pull_from = (((lane_id() & 15) << 2) | (lane_id() >> 4)) << 2;
   auto mma = [&]() {
+    if (transpose_a) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < NA; ++i) a[u][i] = fragment_from_row_order(a[u][i], pull_from);
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -662,7 +695,9 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
   for (; s < ksteps; ++s) {  // remainder when ksteps is not a multiple of U
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      const uint4 av = ld16_once(ap[i] + static_cast<size_t>(s) * astep);
+      uint4 av = transpose_a ? ld16(ap[i] + static_cast<size_t>(s) * astep)
+                             : ld16_once(ap[i] + static_cast<size_t>(s) * astep);
+      if (transpose_a) av = fragment_from_row_order(av, pull_from);
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
         const typename DT::elem* q = bp[r] + static_cast<size_t>(s) * KS;
@@ -773,12 +808,14 @@ __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk
   } else {
     const elem* w13 = reinterpret_cast<const elem*>(p.ffn1) +
                       static_cast<size_t>(tile.expert) * 2 * p.I * p.H;
+    const int wr = row_order_row(), wc = row_order_chunk();
 #pragma unroll
     for (int b = 0; b < G1_NB; ++b) {
-      ap[b] = w13 + static_cast<size_t>(n0 + 16 * b + r16) * p.H + g * EPV;                // gate
-      ap[G1_NB + b] = w13 + static_cast<size_t>(p.I + n0 + 16 * b + r16) * p.H + g * EPV;  // up
+      ap[b] = w13 + static_cast<size_t>(n0 + 16 * b + wr) * p.H + wc * EPV;                // gate
+      ap[G1_NB + b] = w13 + static_cast<size_t>(p.I + n0 + 16 * b + wr) * p.H + wc * EPV;  // up
     }
   }
+  const bool row_major = p.ffn1_packed == nullptr;
   const elem* bp[RB];
   auto token_rows = [&] {
 #pragma unroll
@@ -796,7 +833,7 @@ __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk
     for (int r = 0; r < RB; ++r) acc[i][r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   int status = 0;
-  const bool ran = stream_mma<DT, NA, RB, U, false>(ap, bp, p.H / (4 * EPV), astep, acc, [&] {
+  auto before_rows = [&] {
     if (EARLY) {
       if (!wait_flag(p, FLAG_ROUTED, lds_flag, lds_poller)) {
         status = 1;
@@ -814,7 +851,11 @@ __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk
         bp[r] = reinterpret_cast<const elem*>(p.tokens) + static_cast<size_t>(entry[r] / p.K) * p.H + g * EPV;
     }
     return true;
-  });
+  };
+  // (two instantiations: a run-time switch inside the sweep cost the packed path 6 %)
+  const bool ran = row_major
+                       ? stream_mma<DT, NA, RB, U, false, true>(ap, bp, p.H / (4 * EPV), astep, acc, before_rows)
+                       : stream_mma<DT, NA, RB, U, false, false>(ap, bp, p.H / (4 * EPV), astep, acc, before_rows);
   if (!ran) return status;
 
 #pragma unroll
@@ -905,10 +946,12 @@ __device__ __noinline__ bool down_task(ParamsRef pv, int expert, int row0, int r
   } else {
     const elem* w2 =
         reinterpret_cast<const elem*>(p.ffn2) + static_cast<size_t>(tile.expert) * p.H * p.I;
+    const int wr = row_order_row(), wc = row_order_chunk();
 #pragma unroll
     for (int b = 0; b < NA; ++b)
-      ap[b] = w2 + static_cast<size_t>(n0 + 16 * b + r16) * p.I + g * EPV;
+      ap[b] = w2 + static_cast<size_t>(n0 + 16 * b + wr) * p.I + wc * EPV;
   }
+  const bool row_major = p.ffn2_packed == nullptr;
   // the part of h this tile reads (uniform; the offsets inside it fit 32 bits)
   const size_t hrow0 = static_cast<size_t>(tile.row0);
   const elem* hbase = uniform_ptr(reinterpret_cast<const elem*>(p.h) + hrow0 * p.I);
@@ -940,9 +983,11 @@ __device__ __noinline__ bool down_task(ParamsRef pv, int expert, int row0, int r
   // The h rows are read at agent scope: two gate/up tasks, possibly on different
   // XCDs, each write half of a 128-byte line of h, so this XCD's L2 may hold a
   // line one of its own tasks wrote before the other half existed.
-  const bool ok = stream_mma<DT, NA, RB, U, true>(ap, bp, p.I / (4 * EPV), astep, acc, [&] {
-    return wave_wait_ge(dep, dep_target, p.ctl, p.spin_limit);
-  }, hbase, hbytes);
+  auto wait_for_rows = [&] { return wave_wait_ge(dep, dep_target, p.ctl, p.spin_limit); };
+  const bool ok = row_major ? stream_mma<DT, NA, RB, U, true, true>(ap, bp, p.I / (4 * EPV), astep, acc,
+                                                                     wait_for_rows, hbase, hbytes)
+                            : stream_mma<DT, NA, RB, U, true, false>(ap, bp, p.I / (4 * EPV), astep, acc,
+                                                                      wait_for_rows, hbase, hbytes);
   if (!ok) return false;
 
   float* const ybase = p.y + n0 + 4 * g;

@@ -7,8 +7,8 @@
 // float32 (the reference checks for float32, pyMoeLauncherTorch.cpp:28-29);
 // `create` reads E, H, I and the dtype off the tensors and goes through
 // CreateLauncherEx, with optional top_k (default 8, the reference's compile-time
-// value), router_bias, sched, flags, norm_weight and norm_eps; rank / world_size other than 0 / 1
-// are refused. torch supplies device pointers and the current stream, nothing
+// value), router_bias, sched, flags (left out: a packed copy of the expert weights is kept, see
+// create), norm_weight and norm_eps; rank / world_size other than 0 / 1 are refused. torch supplies device pointers and the current stream, nothing
 // else.
 #include <ATen/hip/HIPContext.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
@@ -53,8 +53,12 @@ class Launcher {
 
   void create(const at::Tensor& gate, const at::Tensor& ffn1, const at::Tensor& ffn2, int max_tokens,
               const py::bytes& uid, int rank, int world_size, int top_k,
-              const c10::optional<at::Tensor>& router_bias, int sched, int flags,
+              const c10::optional<at::Tensor>& router_bias, int sched, const py::object& flags_arg,
               const c10::optional<at::Tensor>& norm_weight, double norm_eps) {
+    // flags left out, as in a call written against the reference: the launcher keeps a packed
+    // copy of the expert weights (the layout the kernels read at full rate; +3*E*H*I elements
+    // of device memory, announced once per process). flags=0 reads the row-major tensors.
+    const int flags = flags_arg.is_none() ? static_cast<int>(FLASH_MOE_FLAG_PACK_WEIGHTS) : flags_arg.cast<int>();
     TORCH_CHECK(impl_ == nullptr, "Launcher already created");
     TORCH_CHECK(gate.defined() && ffn1.defined() && ffn2.defined(), "weight tensor is undefined");
     TORCH_CHECK(gate.dim() == 2 && ffn1.dim() == 3 && ffn2.dim() == 3,
@@ -190,7 +194,7 @@ PYBIND11_MODULE(flashMoeLauncher, m) {
       .def("create", &Launcher::create, py::arg("gate_weights"), py::arg("ffn1_expert_weights"),
            py::arg("ffn2_expert_weights"), py::arg("max_tokens"), py::arg("uid"), py::arg("rank"),
            py::arg("world_size"), py::arg("top_k") = 8, py::arg("router_bias") = py::none(),
-           py::arg("sched") = static_cast<int>(FLASH_MOE_SCHED_AUTO), py::arg("flags") = 0,
+           py::arg("sched") = static_cast<int>(FLASH_MOE_SCHED_AUTO), py::arg("flags") = py::none(),
            py::arg("norm_weight") = py::none(), py::arg("norm_eps") = 1e-6)
       .def("launch", &Launcher::launch, py::arg("tokens"), py::arg("output"))
       .def("destroy", &Launcher::destroy)

@@ -61,9 +61,13 @@ class MoeKernelLauncher:
 
     def create(self, gate_weights, ffn1_expert_weights, ffn2_expert_weights, max_tokens, uid,
                rank, world_size, top_k=8, router_bias=None, sched=_lib.SCHED_AUTO,
-               pack_weights=False, prepacked=False, norm_weight=None, norm_eps=1e-6, residual=False):
-        """norm_weight ([H], the weights' dtype): the layer runs on rmsnorm(tokens) with this
-        weight and norm_eps; residual: the input rows are added to the output."""
+               pack_weights=None, prepacked=False, norm_weight=None, norm_eps=1e-6, residual=False):
+        """pack_weights left out (as in a call written against the reference): the launcher keeps
+        a packed copy of the expert weights, unless they are prepacked; False reads the row-major
+        tensors. norm_weight ([H], the weights' dtype): the layer runs on rmsnorm(tokens) with
+        this weight and norm_eps; residual: the input rows are added to the output."""
+        if pack_weights is None:
+            pack_weights = not prepacked
         _check(self._h is None, "Launcher already created")
         for t, n in ((gate_weights, "gate_weights"), (ffn1_expert_weights, "ffn1_expert_weights"),
                      (ffn2_expert_weights, "ffn2_expert_weights")):

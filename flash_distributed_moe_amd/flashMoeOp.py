@@ -15,7 +15,10 @@ bias are taken from the block when it has them; a launch is one kernel, so
 wrapped block itself (the reference calls `super().forward`, which
 `torch.nn.Module` does not define). `pack_weights` says how the kernels get the
 packed weight layout they read fastest: True (default) keeps a packed second
-copy inside the launcher and leaves the block's tensors alone; "in_place"
+copy inside the launcher and leaves the block's tensors alone (that doubles the
+memory of the block's expert weights: 1.1 GiB per layer of the 30B model, which
+the library announces once per process; a 288 GB device holds the 30B model's 48
+layers twice over, and the block stays usable as the fallback); "in_place"
 rewrites the block's `w13_weight` / `w2_weight` into the packed layout where they
 lie (no extra memory; the wrapped block can then no longer compute with them, so
 `maxTokens` must cover every batch); False reads the row-major tensors.

@@ -13,7 +13,7 @@ from tests.moe_case import GpuCase
 pytestmark = pytest.mark.gpu
 
 CASES = [("tiny_f32", 16, _lib.SCHED_STREAM), ("qwen3_30b_decode", 24, _lib.SCHED_STREAM),
-         ("qwen3_30b_decode", 130, _lib.SCHED_AUTO), ("qwen3_30b_decode", 700, _lib.SCHED_TILED)]
+         ("qwen3_30b_decode", 130, _lib.SCHED_TILED), ("qwen3_30b_decode", 700, _lib.SCHED_TILED)]
 
 
 def _gamma(cfg, dev):

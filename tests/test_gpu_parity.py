@@ -50,19 +50,19 @@ def test_tiny_f32_matches_golden(golden_dir):
         case.close()
 
 
-# AUTO on the caller's weight layout takes the tiled variant from T*k >= 4*E on
+# AUTO takes the streaming variant at this size; the tiled one is asked for by name
 @pytest.mark.parametrize("seed,sched", [(7907, _lib.SCHED_STREAM), (1, _lib.SCHED_STREAM),
-                                        (2, _lib.SCHED_STREAM), (7907, _lib.SCHED_AUTO)])
+                                        (2, _lib.SCHED_STREAM), (7907, _lib.SCHED_AUTO), (7907, _lib.SCHED_TILED)])
 def test_qwen3_30b_decode(seed, sched):
     run_case(synth.CONFIGS["qwen3_30b_decode"], seed=seed, sched=sched)
 
 
-@pytest.mark.parametrize("sched", [_lib.SCHED_STREAM, _lib.SCHED_AUTO])
+@pytest.mark.parametrize("sched", [_lib.SCHED_STREAM, _lib.SCHED_TILED])
 def test_qwen3_30b_decode_inplace(sched):
     run_case(synth.CONFIGS["qwen3_30b_decode"], inplace=True, sched=sched)
 
 
-@pytest.mark.parametrize("sched", [_lib.SCHED_STREAM, _lib.SCHED_AUTO])
+@pytest.mark.parametrize("sched", [_lib.SCHED_STREAM, _lib.SCHED_TILED])
 @pytest.mark.parametrize("T", [1, 3, 17, 65, 130])
 def test_ragged_token_counts_bf16(T, sched):
     cfg = synth.CONFIGS["qwen3_30b_decode"].replace(T=T, name="ragged")
