@@ -65,6 +65,14 @@ enum { FLASH_MOE_FLAG_PACK_WEIGHTS = 1, FLASH_MOE_FLAG_WEIGHTS_PREPACKED = 2 };
  *      of tokens: xn[t,k] = (x[t,k] * float(1/sqrt(mean_k x[t,k]^2 + norm_eps))) *
  *      norm_weight[k], rounded to the layer dtype. A small kernel in front of the
  *      layer's kernel writes xn into the workspace (+max_tokens*H elements).
+ *      The mean of squares is taken in double. For bfloat16 rows that sum is exact
+ *      in any order, so xn (and the routing after it) is reproducible bit for bit
+ *      by a CPU restatement. For float32 rows the squares are exact in double but
+ *      their sum is rounded at every addition, in the kernel's order (64 strided
+ *      partial sums, then a butterfly across the wave): another order can differ
+ *      in the last bits of the double, which changes the float scale only when it
+ *      lies within about 2^-29 ulp of a rounding boundary (about one row in 10^8);
+ *      such a row's xn differs by one float ulp from the restatement's.
  *  FLASH_MOE_FLAG_RESIDUAL  output = tokens + layer(...): the un-normalised input
  *      row is added to the sum over the slots (last, in float) before the one
  *      rounding to the layer dtype. Works in place like everything else.
