@@ -108,7 +108,7 @@ __device__ __forceinline__ TileDesc ld_tile(const TileDesc* t) {
   d.expert = static_cast<int>(v.x);
   d.row0 = static_cast<int>(v.y);
   d.rows = static_cast<int>(v.z);
-  d.pad = 0;
+  d.shared = static_cast<int>(v.w);
   return d;
 }
 

@@ -262,8 +262,16 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   p.bias = d.router_bias;
   const bool pack = (d.flags & FLASH_MOE_FLAG_PACK_WEIGHTS) != 0;
   const bool prepacked = (d.flags & FLASH_MOE_FLAG_WEIGHTS_PREPACKED) != 0;
-  p.ffn1_packed = pack ? l->ws + L.pack1 : prepacked ? d.ffn1_weights : nullptr;
-  p.ffn2_packed = pack ? l->ws + L.pack2 : prepacked ? d.ffn2_weights : nullptr;
+  // A launcher with its own packed copy has both forms and picks per launch. float32 batches
+  // with 16 or more rows an expert run faster on the row-major tensors (30B shape, us,
+  // row-major / packed: T=128 538 / 473, T=192 615 / 565, T=256 592 / 627, T=512 845 / 1088,
+  // T=8192 6770 / 10930: the streaming variant's row tiles of one expert each fetch its
+  // weights again, and the row-major rows stream at the higher rate then); bf16 batches are
+  // faster on the packed copy at every size.
+  const bool use_packed = pack && !(d.dtype == FLASH_MOE_F32 &&
+                                    static_cast<long long>(T) * d.top_k >= 16ll * d.experts);
+  p.ffn1_packed = use_packed ? l->ws + L.pack1 : prepacked ? d.ffn1_weights : nullptr;
+  p.ffn2_packed = use_packed ? l->ws + L.pack2 : prepacked ? d.ffn2_weights : nullptr;
   if (prepacked) p.ffn1 = p.ffn2 = nullptr;  // no row-major form exists
   p.out = output;
   char* w = l->ws;

@@ -65,7 +65,7 @@ struct TileDesc {  // one row tile: `rows` consecutive permuted rows of one expe
   int expert;
   int row0;
   int rows;
-  int pad;
+  int shared;  // streaming variant: the expert has other row tiles, which read the same weights
 };
 
 // One record per executed task when tracing is on (times: 100 MHz wall clock).

@@ -370,7 +370,7 @@ __device__ __noinline__ void scan_task(ParamsRef pv) {
         if (toff + i < r.max_mtiles) {
           stc16(&r.mtiles[toff + i],
                 make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + i * SKINNY_MT),
-                           static_cast<unsigned>(min(SKINNY_MT, c - i * SKINNY_MT)), 0u));
+                           static_cast<unsigned>(min(SKINNY_MT, c - i * SKINNY_MT)), nt > 1 ? 1u : 0u));
         }
       }
     }
@@ -492,7 +492,8 @@ __device__ __noinline__ void scan_scatter_small_task(ParamsRef pv) {
         if (toff + i < r.max_mtiles) {
           stc16(&r.mtiles[toff + i],
                 make_uint4(static_cast<unsigned>(e), static_cast<unsigned>(off + i * SKINNY_MT),
-                           static_cast<unsigned>(p.early ? c : min(SKINNY_MT, c - i * SKINNY_MT)), 0u));
+                           static_cast<unsigned>(p.early ? c : min(SKINNY_MT, c - i * SKINNY_MT)),
+                           c > SKINNY_MT ? 1u : 0u));
         }
       }
     }
@@ -615,7 +616,7 @@ __device__ __forceinline__ uint4 fragment_from_row_order(const uint4& v, int pul
 __device__ __forceinline__ int row_order_row() { return lane_id() >> 2; }
 __device__ __forceinline__ int row_order_chunk() { return lane_id() & 3; }
 
-template <typename DT, int NA, int RB, int U, bool COH_B, bool transpose_a, typename Pre>
+template <typename DT, int NA, int RB, int U, bool COH_B, bool transpose_a, bool once_a, typename Pre>
 __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[NA],
                                            const typename DT::elem* const (&bp)[RB], int ksteps,
                                            int astep, f32x4 (&acc)[NA][RB], Pre pre,
@@ -640,11 +641,15 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int i = 0; i < NA; ++i) {
-        // row-major rows are read half a line at a time: the other half comes with the next
-        // k-step and must find the line still cached, so these loads are ordinary ones (with
-        // the non-temporal hint the second half was fetched again: 64 tokens 300 -> 273 us)
-        a[u][i] = transpose_a ? ld16(ap[i] + static_cast<size_t>(s + u) * astep)
-                              : ld16_once(ap[i] + static_cast<size_t>(s + u) * astep);
+        // once_a: the weights have no other reader in this launch, so they pass through the
+        // caches without staying (non-temporal). Not for row-major rows, which are read half a
+        // line at a time: the other half comes with the next k-step and must find the line still
+        // cached (with the hint it was fetched again: 64 tokens 300 -> 273 us). Not for an
+        // expert with several row tiles either, whose tasks read the same weights at about the
+        // same time (bf16, 30B shape, streaming variant forced: 1024 tokens 538 -> 485 us, 4096
+        // tokens 1638 -> 1433 us with ordinary loads).
+        a[u][i] = once_a ? ld16_once(ap[i] + static_cast<size_t>(s + u) * astep)
+                         : ld16(ap[i] + static_cast<size_t>(s + u) * astep);
       }
   };
   auto load_b = [&](int s) {
@@ -695,8 +700,8 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
   for (; s < ksteps; ++s) {  // remainder when ksteps is not a multiple of U
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      uint4 av = transpose_a ? ld16(ap[i] + static_cast<size_t>(s) * astep)
-                             : ld16_once(ap[i] + static_cast<size_t>(s) * astep);
+      uint4 av = once_a ? ld16_once(ap[i] + static_cast<size_t>(s) * astep)
+                        : ld16(ap[i] + static_cast<size_t>(s) * astep);
       if (transpose_a) av = fragment_from_row_order(av, pull_from);
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
@@ -853,9 +858,11 @@ __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk
     return true;
   };
   // (two instantiations: a run-time switch inside the sweep cost the packed path 6 %)
-  const bool ran = row_major
-                       ? stream_mma<DT, NA, RB, U, false, true>(ap, bp, p.H / (4 * EPV), astep, acc, before_rows)
-                       : stream_mma<DT, NA, RB, U, false, false>(ap, bp, p.H / (4 * EPV), astep, acc, before_rows);
+  const bool ran =
+      row_major ? stream_mma<DT, NA, RB, U, false, true, false>(ap, bp, p.H / (4 * EPV), astep, acc, before_rows)
+      : tile.shared != 0
+          ? stream_mma<DT, NA, RB, U, false, false, false>(ap, bp, p.H / (4 * EPV), astep, acc, before_rows)
+          : stream_mma<DT, NA, RB, U, false, false, true>(ap, bp, p.H / (4 * EPV), astep, acc, before_rows);
   if (!ran) return status;
 
 #pragma unroll
@@ -885,7 +892,7 @@ __device__ __forceinline__ int gateup_body(ParamsRef p, TileDesc& tile, int nblk
 }
 
 template <typename DT, int RB>
-__device__ __noinline__ void gateup_task(ParamsRef pv, int expert, int row0, int rows, int nblk) {
+__device__ __noinline__ void gateup_task(ParamsRef pv, int expert, int row0, int rows, int nblk, int shared) {
   // (the row tile arrives as three integers: a struct by value makes the callee save
   // and restore every callee-saved register it touches, a struct by reference costs
   // a trip to the caller's private memory)
@@ -894,7 +901,7 @@ __device__ __noinline__ void gateup_task(ParamsRef pv, int expert, int row0, int
   tile.expert = expert;
   tile.row0 = row0;
   tile.rows = rows;
-  tile.pad = 0;
+  tile.shared = __builtin_amdgcn_readfirstlane(shared);
   gateup_body<DT, RB, false>(p, tile, nblk, nullptr, nullptr);
 }
 
@@ -907,7 +914,7 @@ __device__ __noinline__ int gateup_early_task(ParamsRef pv, int expert, int nblk
   tile.expert = expert;
   tile.row0 = 0;
   tile.rows = 0;
-  tile.pad = 0;
+  tile.shared = 0;
   return gateup_body<DT, RB, true>(p, tile, nblk, lds_flag, lds_poller);
 }
 
@@ -918,14 +925,14 @@ __device__ __noinline__ int gateup_early_task(ParamsRef pv, int expert, int nblk
 // on h, so their first loads are issued before the wait for the tile's
 // gate/up tasks. Returns false if that wait failed.
 template <typename DT, int RB>
-__device__ __noinline__ bool down_task(ParamsRef pv, int expert, int row0, int rows, int nblk,
+__device__ __noinline__ bool down_task(ParamsRef pv, int expert, int row0, int rows, int nblk, int shared,
                                        unsigned* dep, unsigned dep_target) {
   ParamsRef p = uniform_params(pv);
   TileDesc tile;
   tile.expert = expert;
   tile.row0 = row0;
   tile.rows = rows;
-  tile.pad = 0;
+  tile.shared = __builtin_amdgcn_readfirstlane(shared);
   typedef typename DT::elem elem;
   constexpr int EPV = DT::EPV;
   constexpr int NA = G2_NB;
@@ -984,10 +991,14 @@ __device__ __noinline__ bool down_task(ParamsRef pv, int expert, int row0, int r
   // XCDs, each write half of a 128-byte line of h, so this XCD's L2 may hold a
   // line one of its own tasks wrote before the other half existed.
   auto wait_for_rows = [&] { return wave_wait_ge(dep, dep_target, p.ctl, p.spin_limit); };
-  const bool ok = row_major ? stream_mma<DT, NA, RB, U, true, true>(ap, bp, p.I / (4 * EPV), astep, acc,
-                                                                     wait_for_rows, hbase, hbytes)
-                            : stream_mma<DT, NA, RB, U, true, false>(ap, bp, p.I / (4 * EPV), astep, acc,
-                                                                      wait_for_rows, hbase, hbytes);
+  const bool ok =
+      row_major ? stream_mma<DT, NA, RB, U, true, true, false>(ap, bp, p.I / (4 * EPV), astep, acc, wait_for_rows,
+                                                               hbase, hbytes)
+      : tile.shared != 0
+          ? stream_mma<DT, NA, RB, U, true, false, false>(ap, bp, p.I / (4 * EPV), astep, acc, wait_for_rows,
+                                                          hbase, hbytes)
+          : stream_mma<DT, NA, RB, U, true, false, true>(ap, bp, p.I / (4 * EPV), astep, acc, wait_for_rows,
+                                                         hbase, hbytes);
   if (!ok) return false;
 
   float* const ybase = p.y + n0 + 4 * g;
@@ -1267,7 +1278,7 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
         tile.expert = static_cast<int>(aux);
         tile.row0 = 0;
         tile.rows = 0;
-        tile.pad = 0;
+        tile.shared = 0;
         // (p.early is the number of 16-row blocks an early task carries)
         const int st = p.early == 1
                            ? gateup_early_task<DT, 1>(p, tile.expert, nblk, lds_flag, lds_poller)
@@ -1282,11 +1293,11 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
           for (int r0 = 0; r0 < tile.rows; r0 += SKINNY_MT) {
             const int rc = min(SKINNY_MT, tile.rows - r0);
             if (rc <= 16) {
-              gateup_task<DT, 1>(p, tile.expert, tile.row0 + r0, rc, nblk);
+              gateup_task<DT, 1>(p, tile.expert, tile.row0 + r0, rc, nblk, 1);
             } else if (rc <= 32) {
-              gateup_task<DT, 2>(p, tile.expert, tile.row0 + r0, rc, nblk);
+              gateup_task<DT, 2>(p, tile.expert, tile.row0 + r0, rc, nblk, 1);
             } else {
-              gateup_task<DT, 4>(p, tile.expert, tile.row0 + r0, rc, nblk);
+              gateup_task<DT, 4>(p, tile.expert, tile.row0 + r0, rc, nblk, 1);
             }
           }
         }
@@ -1302,11 +1313,11 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
         const TileDesc tile = ld_tile(&p.mtiles[aux]);
         const int nblk = static_cast<int>(j % nt1);
         if (tile.rows <= 16) {
-          gateup_task<DT, 1>(p, tile.expert, tile.row0, tile.rows, nblk);
+          gateup_task<DT, 1>(p, tile.expert, tile.row0, tile.rows, nblk, tile.shared);
         } else if (tile.rows <= 32) {
-          gateup_task<DT, 2>(p, tile.expert, tile.row0, tile.rows, nblk);
+          gateup_task<DT, 2>(p, tile.expert, tile.row0, tile.rows, nblk, tile.shared);
         } else {
-          gateup_task<DT, 4>(p, tile.expert, tile.row0, tile.rows, nblk);
+          gateup_task<DT, 4>(p, tile.expert, tile.row0, tile.rows, nblk, tile.shared);
         }
         wave_arrive(&p.g1_done[aux].v);
       } else if (j < n1 + n2) {
@@ -1332,21 +1343,21 @@ __global__ __launch_bounds__(512) __attribute__((disable_tail_calls)) void moe_s
           if (tile.rows == 0) {
             ok = true;
           } else if (tile.rows <= 16) {
-            ok = down_task<DT, 1>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
+            ok = down_task<DT, 1>(p, tile.expert, tile.row0, tile.rows, nblk, tile.shared, dep, nt1);
           } else if (tile.rows <= 32) {
-            ok = down_task<DT, 2>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
+            ok = down_task<DT, 2>(p, tile.expert, tile.row0, tile.rows, nblk, tile.shared, dep, nt1);
           } else if (tile.rows <= SKINNY_MT) {
-            ok = down_task<DT, 4>(p, tile.expert, tile.row0, tile.rows, nblk, dep, nt1);
+            ok = down_task<DT, 4>(p, tile.expert, tile.row0, tile.rows, nblk, tile.shared, dep, nt1);
           } else {
             ok = true;
             for (int r0 = 0; ok && r0 < tile.rows; r0 += SKINNY_MT) {
               const int rc = min(SKINNY_MT, tile.rows - r0);
               if (rc <= 16) {
-                ok = down_task<DT, 1>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+                ok = down_task<DT, 1>(p, tile.expert, tile.row0 + r0, rc, nblk, 1, dep, nt1);
               } else if (rc <= 32) {
-                ok = down_task<DT, 2>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+                ok = down_task<DT, 2>(p, tile.expert, tile.row0 + r0, rc, nblk, 1, dep, nt1);
               } else {
-                ok = down_task<DT, 4>(p, tile.expert, tile.row0 + r0, rc, nblk, dep, nt1);
+                ok = down_task<DT, 4>(p, tile.expert, tile.row0 + r0, rc, nblk, 1, dep, nt1);
               }
             }
           }

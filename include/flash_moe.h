@@ -49,8 +49,9 @@ enum { FLASH_MOE_SCHED_AUTO = 0, FLASH_MOE_SCHED_STREAM = 1, FLASH_MOE_SCHED_TIL
  *  FLASH_MOE_FLAG_PACK_WEIGHTS      at create the library copies the caller's
  *      row-major expert weights into a packed second copy in its workspace
  *      (+3*E*H*I elements of device memory). The caller's tensors stay the external
- *      format and are no longer read by launches; after changing them call
- *      flashMoeRefreshWeights.
+ *      format and must stay valid: a launch reads whichever form is faster for its
+ *      batch (bf16: always the copy; float32: the caller's tensors from 16 rows an
+ *      expert on). After changing them call flashMoeRefreshWeights.
  *  FLASH_MOE_FLAG_WEIGHTS_PREPACKED ffn1_weights / ffn2_weights already hold the
  *      packed layout (made by flashMoePackWeights into buffers of the caller's, or
  *      by flashMoePackWeightsInPlace): no second copy anywhere; the row-major form

@@ -32,7 +32,7 @@ _first_output = {}   # (config, T) -> output of the first variant run: later var
 
 
 def run_full(name, T=None, pack_weights=False, same_bits_as_first=False, fresh_relaunch=False):
-    cfg = synth.CONFIGS[name]
+    cfg = synth.CONFIGS[name] if isinstance(name, str) else name
     if T is not None:
         cfg = cfg.replace(T=T)
     print("full config", cfg.name, "T", cfg.T, "packed" if pack_weights else "caller's layout", flush=True)
@@ -123,3 +123,13 @@ def test_qwen3_30b_imbalance():
     share = r["counts"][hot].sum() / r["counts"].sum()
     print("  hot experts", hot, "share %.3f" % share, flush=True)
     assert 0.40 < share <= 0.5001                     # the 4 biased experts take about half
+
+
+@pytest.mark.parametrize("pack_weights", [False, True])
+def test_f32_30b_large_batch(pack_weights):
+    """The reference's own dtype and shape (src/hip/common/metadata.h:7-13) at a batch its GPU
+    path cannot hold (capacity about 85 tokens, src/hip/moeKernelLauncher.hip:117-135): the
+    streaming variant with several row tiles an expert. With its own packed copy the
+    launcher reads the row-major tensors at this size (legacy CreateLauncher's case)."""
+    cfg = synth.MoeConfig("f32_30b_t1024", 1024, 2048, 128, 8, 768, "f32")
+    run_full(cfg, pack_weights=pack_weights, same_bits_as_first=True, fresh_relaunch=not pack_weights)

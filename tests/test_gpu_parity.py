@@ -236,7 +236,10 @@ def test_packed_weights_equal_unpacked(name, T):
 
 @pytest.mark.parametrize("name,T,sched", [("qwen3_30b_decode", 64, _lib.SCHED_STREAM),
                                           ("qwen3_30b_decode", 700, _lib.SCHED_TILED),
-                                          ("tiny_f32", 16, _lib.SCHED_STREAM)])
+                                          ("tiny_f32", 16, _lib.SCHED_STREAM),
+                                          # several row tiles an expert: their tasks share the weights
+                                          ("qwen3_30b_decode", 1500, _lib.SCHED_STREAM),
+                                          ("tiny_f32", 600, _lib.SCHED_STREAM)])
 def test_prepacked_weights_equal_unpacked(name, T, sched):
     """Weights packed in place by the caller (no second copy anywhere, the
     launcher's workspace holds no weight-sized region) give the same bits as the
