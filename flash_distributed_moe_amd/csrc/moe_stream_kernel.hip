@@ -662,21 +662,35 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
       }
   };
   const int pull_from = (((lane_id() & 15) << 2) | (lane_id() >> 4)) << 2;
-  auto mma = [&]() {
+  auto load_step = [&](int u, int s) {  // the loads of k-step s into slot u
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+      a[u][i] = once_a ? ld16_once(ap[i] + static_cast<size_t>(s) * astep)
+                       : ld16(ap[i] + static_cast<size_t>(s) * astep);
+#pragma unroll
+    for (int r = 0; r < RB; ++r) b[u][r] = ld_b(bp[r] + static_cast<size_t>(s) * KS);
+  };
+  auto mma_step = [&](int u) {
     if (transpose_a) {
 #pragma unroll
-      for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int i = 0; i < NA; ++i) a[u][i] = fragment_from_row_order(a[u][i], pull_from);
+      for (int i = 0; i < NA; ++i) a[u][i] = fragment_from_row_order(a[u][i], pull_from);
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int i = 0; i < NA; ++i)
 #pragma unroll
-      for (int i = 0; i < NA; ++i)
-#pragma unroll
-        for (int r = 0; r < RB; ++r) acc[i][r] = mma16<DT>(a[u][i], b[u][r], acc[i][r]);
+      for (int r = 0; r < RB; ++r) acc[i][r] = mma16<DT>(a[u][i], b[u][r], acc[i][r]);
   };
 
+  // One block of 16 rows (ROLL): the window of U k-steps is filled once; from then on a slot
+  // is asked for again as soon as its matrix instructions have read it, so the wave keeps
+  // U - 1 steps' loads in flight all the time instead of a burst per round that drains
+  // before the next one. With more row blocks the window is shorter (U = 4) and the bursts
+  // do better.
+  constexpr bool ROLL = RB == 1;
+  auto mma = [&]() {
+#pragma unroll
+    for (int u = 0; u < U; ++u) mma_step(u);
+  };
   const int main_steps = (ksteps / U) * U;
   int s = 0;
   if (main_steps > 0) {
@@ -685,17 +699,31 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
     if (!pre()) return false;
     load_b(0);
     __builtin_amdgcn_sched_barrier(0);
-    mma();
-    s = U;
+    if constexpr (ROLL) {
+      for (; s + 2 * U <= main_steps; s += U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          mma_step(u);
+          __builtin_amdgcn_sched_barrier(0);
+          load_step(u, s + U + u);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      mma();
+      s += U;
+    } else {
+      mma();
+      s = U;
+      for (; s < main_steps; s += U) {
+        __builtin_amdgcn_sched_barrier(0);
+        load_a(s);
+        load_b(s);
+        __builtin_amdgcn_sched_barrier(0);
+        mma();
+      }
+    }
   } else {
     if (!pre()) return false;
-  }
-  for (; s < main_steps; s += U) {
-    __builtin_amdgcn_sched_barrier(0);
-    load_a(s);
-    load_b(s);
-    __builtin_amdgcn_sched_barrier(0);
-    mma();
   }
   for (; s < ksteps; ++s) {  // remainder when ksteps is not a multiple of U
 #pragma unroll
