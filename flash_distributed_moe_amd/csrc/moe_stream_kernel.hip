@@ -684,8 +684,9 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
   // One block of 16 rows (ROLL): the window of U k-steps is filled once; from then on a slot
   // is asked for again as soon as its matrix instructions have read it, so the wave keeps
   // U - 1 steps' loads in flight all the time instead of a burst per round that drains
-  // before the next one. With more row blocks the window is shorter (U = 4) and the bursts
-  // do better.
+  // before the next one (a bare read loop of the same loads on all CUs: 4.7 TB/s in bursts,
+  // 6.3 TB/s refilled slot by slot). With more row blocks the bursts do better (two blocks:
+  // 256 tokens 272 -> 275 us, 235B shape 853 -> 867 us with refills).
   constexpr bool ROLL = RB == 1;
   auto mma = [&]() {
 #pragma unroll
@@ -700,7 +701,7 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
     load_b(0);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (ROLL) {
-      for (; s + 2 * U <= main_steps; s += U) {
+      auto round = [&]() {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           mma_step(u);
@@ -708,6 +709,17 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
           load_step(u, s + U + u);
           __builtin_amdgcn_sched_barrier(0);
         }
+        s += U;
+      };
+      // The first round stands in front of the loop: the window's first loads were issued
+      // operand by operand (every weight load, then every token load), later ones step by
+      // step, and the compiler counts the loads a step may leave in flight from both orders
+      // wherever the two meet (with the first round inside the loop every round's first step
+      // waited until 7 loads were left of 40).
+      if (s + 2 * U <= main_steps) {
+        round();
+        asm volatile("; end of the first round" ::: "memory");  // keeps it apart from the loop
+        while (s + 2 * U <= main_steps) round();
       }
       mma();
       s += U;
