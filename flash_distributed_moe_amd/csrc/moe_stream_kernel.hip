@@ -686,8 +686,10 @@ __device__ __forceinline__ bool stream_mma(const typename DT::elem* const (&ap)[
   // U - 1 steps' loads in flight all the time instead of a burst per round that drains
   // before the next one (a bare read loop of the same loads on all CUs: 4.7 TB/s in bursts,
   // 6.3 TB/s refilled slot by slot). With more row blocks the bursts do better (two blocks:
-  // 256 tokens 272 -> 275 us, 235B shape 853 -> 867 us with refills).
-  constexpr bool ROLL = RB == 1;
+  // 256 tokens 272 -> 275 us, 235B shape 853 -> 867 us with refills), and so they do on
+  // row-major weights (64 tokens 272 against 275 us: a line's second half, asked for one
+  // step after the first, misses more often behind a steady stream of other requests).
+  constexpr bool ROLL = RB == 1 && !transpose_a;
   auto mma = [&]() {
 #pragma unroll
     for (int u = 0; u < U; ++u) mma_step(u);
