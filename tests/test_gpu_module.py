@@ -175,3 +175,38 @@ def test_wrapper_packs_the_blocks_weights_in_place():
     with pytest.raises(RuntimeError, match="packed in place"):
         layer(torch.cat([x, x], 0))
     del layer, plain
+
+
+@pytest.mark.parametrize("name,T", [("qwen3_30b_decode", 64), ("qwen3_30b_decode", 700), ("tiny_f32", 16)])
+def test_extension_and_ctypes_mirror_agree(name, T):
+    """The compiled `flashMoeLauncher` extension (what callers import) and the ctypes class the
+    parity tests drive end in the same C entry points: same bits for the same call, with the
+    defaults of both (`create` without flags: the launcher's packed copy), and the same refusals."""
+    import flashMoeLauncher as ext
+    from flash_distributed_moe_amd.flashMoeLauncher import MoeKernelLauncher as Mirror
+
+    cfg = synth.CONFIGS[name].replace(T=T)
+    dev = torch.device("cuda:0")
+    inp = synth.make_inputs_torch(cfg, 31, dev)
+    x = inp["tokens"]
+    outs = []
+    for cls in (ext.MoeKernelLauncher, Mirror):
+        l = cls()
+        uid = l.getDistributedUniqueId(empty=True)
+        assert bytes(uid) == bytes(128)
+        l.create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T, uid, 0, 1, top_k=cfg.k)
+        out = torch.full_like(x, float("nan"))
+        l.launch(x, out)
+        torch.cuda.synchronize()
+        outs.append(out.clone())
+        for bad in (lambda: l.launch(x, out[:1]),                      # shapes differ
+                    lambda: l.launch(x.float() if x.dtype != torch.float32 else x.bfloat16(), out)):  # dtype
+            with pytest.raises((RuntimeError, ValueError, TypeError)):
+                bad()
+        l.destroy()
+        assert not l.valid
+        with pytest.raises(RuntimeError, match="Launcher was destroyed"):
+            l.launch(x, out)
+        with pytest.raises((RuntimeError, ValueError)):
+            cls().create(inp["gate"], inp["ffn1"], inp["ffn2"], cfg.T, uid, 1, 2, top_k=cfg.k)  # world size 2
+    assert torch.equal(outs[0], outs[1])
