@@ -206,6 +206,100 @@ def workgroup_balance(launcher, x, out, tokens, waves_per_group):
             "traced_span_us": span, "tasks": int(len(rec)), "tokens": int(tokens)}
 
 
+def board_power(name, seed, sched, weights, seconds=2.0):
+    """Back-to-back launches of workload `name` for about `seconds`, with the board power the
+    driver reports (hwmon power1_input / power1_average, microwatts) sampled every 20 ms from a
+    thread of this process: what the launch draws against the board's power cap, next to the
+    same reading with the GPU idle."""
+    import glob
+    import threading
+
+    import torch
+
+    from flash_distributed_moe_amd import synth
+    from flash_distributed_moe_amd.flashMoeLauncher import MoeKernelLauncher
+
+    files = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") +
+                   glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"))
+    caps = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"))
+    if not files:
+        sys.exit("bench.py --power: the driver exposes no hwmon power reading here")
+
+    def read(path):
+        try:
+            return int(open(path).read().strip()) / 1e6
+        except (OSError, ValueError):
+            return None
+
+    launcher = None
+    if name == "vendor_gemm_8192":
+        # the vendor's bf16 GEMM (torch.matmul) for comparison: 8192 x 8192 x 8192
+        a = torch.randn(8192, 8192, device="cuda:0", dtype=torch.bfloat16)
+        b = torch.randn(8192, 8192, device="cuda:0", dtype=torch.bfloat16) * 0.02
+
+        def launch():
+            torch.matmul(a, b.t())
+    else:
+        cfg = synth.CONFIGS[name]
+        inp = synth.make_inputs_torch(cfg, seed, torch.device("cuda:0"))
+        x = inp["tokens"]
+        out = torch.empty_like(x)
+        launcher = MoeKernelLauncher()
+        ffn1, ffn2 = inp["ffn1"], inp["ffn2"]
+        if weights == "in_place":
+            ffn1, ffn2 = ffn1.clone(), ffn2.clone()
+            MoeKernelLauncher.pack_weights_in_place(ffn1, ffn2)
+        launcher.create(inp["gate"], ffn1, ffn2, cfg.T, launcher.getDistributedUniqueId(empty=True), 0, 1,
+                        top_k=cfg.k, router_bias=inp["bias"], sched=sched, prepacked=weights == "in_place",
+                        pack_weights={"in_place": False, "default": None, "row_major": False}[weights])
+
+        def launch():
+            launcher.launch(x, out)
+    for _ in range(20):
+        launch()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(50):
+        launch()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / 50
+    launches = max(100, int(seconds * 1e6 / us))
+    time.sleep(1.0)
+
+    samples, stop = [], [False]
+
+    def poll():
+        while not stop[0]:
+            samples.append((time.perf_counter(), read(files[0])))
+            time.sleep(0.02)
+
+    th = threading.Thread(target=poll)
+    th.start()
+    time.sleep(0.4)
+    t0 = time.perf_counter()
+    for _ in range(launches):
+        launch()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    stop[0] = True
+    th.join()
+    if launcher is not None:
+        err, _ = launcher.status()
+        launcher.destroy()
+        if err:
+            sys.exit("bench.py: device error bits %d" % err)
+    idle = [w for t, w in samples if t < t0 - 0.05 and w is not None]
+    busy = [w for t, w in samples if t0 + 0.3 < t < t1 - 0.05 and w is not None]
+    return {"workload": name, "launches": launches, "us_per_launch": (t1 - t0) / launches * 1e6,
+            "power_file": files[0], "samples_busy": len(busy),
+            "power_w_idle": sum(idle) / len(idle) if idle else None,
+            "power_w_busy_mean": sum(busy) / len(busy) if busy else None,
+            "power_w_busy_max": max(busy) if busy else None,
+            "power_cap_w": read(caps[0]) if caps else None}
+
+
 def measure(name, seed, steps, warmup, sched, weights, cold=False, balance=False):
     """K timed launches of workload `name`: whole-job wall time, the kernel's launch-to-launch
     duration from events on the launch stream, and where that puts it on its roofline."""
@@ -324,6 +418,9 @@ def main():
     ap.add_argument("--gemm-calibration", action="store_true",
                     help="time torch.matmul (the vendor GEMM) in bf16 on this box: the matrix-core "
                          "rate reachable in practice, next to the published peak")
+    ap.add_argument("--power", action="store_true",
+                    help="launch --config back to back for two seconds and report the board power "
+                         "the driver reads meanwhile, beside the power cap")
     ap.add_argument("--record-traffic", nargs=2, type=float, metavar=("FETCH_KIB", "WRITE_KIB"),
                     help="no GPU work: write the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings "
                          "(KiB per dispatch) of --config into profiles/traffic.json")
@@ -379,6 +476,10 @@ def main():
                          "frac_of_2500": 2.0 * m * n * k / us / 1e6 / 2500.0}
             del a, b
         print(json.dumps({"gemm_calibration": out}))
+        return
+
+    if args.power:
+        print(json.dumps({"board_power": board_power(args.config, args.seed, args.sched, packed)}))
         return
 
     headline = args.config == "qwen3_30b_decode"
