@@ -62,7 +62,7 @@ def test_topk_ties_nan_short_rows(golden_dir):
     v, i = oracle.topk(g["tie_rows"], 4)
     assert np.array_equal(i, g["tie_idx"])
     assert np.array_equal(v, g["tie_vals"], equal_nan=True)
-    # the survey's probe: {1,3,3,0,3,1,1,-2}, k=4 -> 1 2 4 0
+    # ties by hand: {1,3,3,0,3,1,1,-2}, k=4 -> the three 3s in index order, then the first 1
     assert i[0].tolist() == [1, 2, 4, 0]
     v, i = oracle.topk(g["short_rows"], 5)
     assert np.array_equal(i, g["short_idx"])
