@@ -73,6 +73,12 @@ struct Layout {
 
 constexpr int kMaxGroups = 1024;  // workgroups a launch may use (one per CU)
 
+// AUTO hands a batch to the tiled variant from this many rows an expert on (on average):
+// packed weights / the caller's row-major weights. Below it the streaming variant runs, which
+// is what its share of `y` is sized for.
+constexpr int kAutoTiledRowsPacked = 26;
+constexpr int kAutoTiledRowsRowMajor = 14;
+
 // need_tiled: the tiled variant may run on this workspace.
 Layout make_layout(const FlashMoeLayerDesc& d, bool need_tiled) {
   Layout L{};
@@ -111,7 +117,7 @@ Layout make_layout(const FlashMoeLayerDesc& d, bool need_tiled) {
   const bool tiled_all = need_tiled && static_cast<long long>(d.max_tokens) * d.hidden * 2 < (1ll << 32);
   const size_t stream_rows =
       tiled_all && d.sched == FLASH_MOE_SCHED_TILED ? 0
-      : tiled_all && d.sched == FLASH_MOE_SCHED_AUTO ? std::min<size_t>(rows, 24 * static_cast<size_t>(d.experts))
+      : tiled_all && d.sched == FLASH_MOE_SCHED_AUTO ? std::min<size_t>(rows, kAutoTiledRowsPacked * static_cast<size_t>(d.experts))
                                                      : rows;
   L.y = take(std::max(sizeof(float) * stream_rows * d.hidden,
                       need_tiled ? fmoe::tiled_y_bytes(rows, d.hidden) : 0));
@@ -157,13 +163,13 @@ hipError_t validate(const FlashMoeLayerDesc* d) {
 }
 
 // The tiled variant needs bf16, tile-aligned shapes and token rows it can
-// address with 32-bit byte offsets. AUTO takes it once an expert sees about 22
+// address with 32-bit byte offsets. AUTO takes it once an expert sees about 26
 // rows on average when the weights are packed (30B shape, us, streaming / tiled:
-// T=256 288 / 299, T=320 298 / 299, T=384 306 / 301, T=512 340 / 304; 235B shape:
-// T=256 925 / 952, T=384 985 / 966, T=512 1064 / 977), and from about 14 rows on
+// T=320 284 / 301, T=384 293 / 301, T=448 314 / 299, T=512 339 / 304; 235B shape:
+// T=320 905 / 960, T=384 934 / 969, T=512 1054 / 976), and from about 14 rows on
 // the caller's row-major weights, which the streaming variant reads half a
-// cache line at a time (30B: T=64 272 / 315, T=128 287 / 315, T=192 309 / 316,
-// T=256 319 / 318, T=384 359 / 322; 235B: T=128 961 / 973, T=256 1036 / 996).
+// cache line at a time (30B: T=192 309 / 318, T=256 318 / 318, T=320 346 / 320;
+// 235B: T=192 1030 / 1001, T=256 1055 / 1007, T=384 1142 / 1015).
 bool tiled_eligible(const FlashMoeLayerDesc& d, int tokens_num) {
   return d.dtype == FLASH_MOE_BF16 && d.hidden % 256 == 0 && d.intermediate % 128 == 0 &&
          tokens_num <= fmoe::tiled_max_tokens() &&
@@ -176,7 +182,9 @@ int sched_for(const FlashMoeLayerDesc& d, int tokens_num) {
   if (d.sched == FLASH_MOE_SCHED_TILED) return FLASH_MOE_SCHED_TILED;
   const long long rows = static_cast<long long>(tokens_num) * d.top_k;
   const bool packed = (d.flags & (FLASH_MOE_FLAG_PACK_WEIGHTS | FLASH_MOE_FLAG_WEIGHTS_PREPACKED)) != 0;
-  return rows >= (packed ? 22ll : 14ll) * d.experts ? FLASH_MOE_SCHED_TILED : FLASH_MOE_SCHED_STREAM;
+  return rows >= static_cast<long long>(packed ? kAutoTiledRowsPacked : kAutoTiledRowsRowMajor) * d.experts
+             ? FLASH_MOE_SCHED_TILED
+             : FLASH_MOE_SCHED_STREAM;
 }
 
 // Whether any batch size up to max_tokens may run the tiled variant.
