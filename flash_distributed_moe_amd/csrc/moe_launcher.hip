@@ -249,11 +249,13 @@ fmoe::Params make_params(const FlashMoeLauncher* l, const void* tokens, void* ou
   const bool reaches_experts =
       static_cast<long long>(T) * d.top_k >= static_cast<long long>(d.experts);
   // An early task serves one block of 16 rows, or two; a tile with more starts
-  // over from the tile table once the scan is done. So: one block up to 12 rows
-  // per expert on average (30B shape, with / without: T=80 230 / 243 us, T=128
-  // 242 / 253, T=192 263 / 266), two up to 24.
+  // over from the tile table once the scan is done. So: one block up to 9 rows
+  // per expert on average, two up to 24 (30B shape, us, none / one / two: T=64
+  // 239 / 222 / 226, T=128 257 / 241 / 242, T=160 265 / 259 / 252, T=192 273 / 263 /
+  // 259, T=256 284 / 289 / 272; 235B shape: T=128 821 / 792 / 805, T=192 865 / 850 /
+  // 833, T=256 894 / 942 / 856).
   const long long slots = static_cast<long long>(T) * d.top_k;
-  const int early_blocks = slots <= 12ll * d.experts ? 1 : slots <= 24ll * d.experts ? 2 : 0;
+  const int early_blocks = slots <= 9ll * d.experts ? 1 : slots <= 24ll * d.experts ? 2 : 0;
   p.early = (reaches_experts && early_blocks != 0 && p.fuse_scatter &&
              T <= fmoe::EARLY_MAX_TOKENS &&
              d.experts * ((T + 63) / 64) <= fmoe::SCAN_LDS_WORDS && d.experts <= L.max_mtiles &&
